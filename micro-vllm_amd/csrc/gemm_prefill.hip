@@ -147,8 +147,13 @@ __device__ __forceinline__ void store_wave_tile(const PGemmArgs& a, const f32x4_
         f32x4_t c = acc[i][t];
         for (int e = 0; e < nlower; ++e) {
             f32x4_t part;
+            // the base is the same for every lane; the scalar-register operand needs the compiler to know it
+            const unsigned long long base = (unsigned long long)(lower + (size_t)e * 8 * kWSlotBytes + (i * 8 + t) * 1024);
+            const unsigned long long ubase =
+                ((unsigned long long)__builtin_amdgcn_readfirstlane((unsigned)(base >> 32)) << 32) |
+                (unsigned)__builtin_amdgcn_readfirstlane((unsigned)base);
             asm volatile("global_load_dwordx4 %0, %1, %2 sc1\n\ts_waitcnt vmcnt(0)"
-                         : "=v"(part) : "v"(lane16), "s"(lower + (size_t)e * 8 * kWSlotBytes + (i * 8 + t) * 1024) : "memory");
+                         : "=v"(part) : "v"(lane16), "s"((const unsigned char*)ubase) : "memory");
             c += part;
         }
         return c;
