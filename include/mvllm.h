@@ -455,6 +455,91 @@ int mv_graph_end_capture(mv_stream_t stream, void** graph_exec_out);
 int mv_graph_launch(void* graph_exec, mv_stream_t stream);
 int mv_graph_destroy(void* graph_exec);
 
+/* ------------------------------------------------------------------------------------------------
+ * Layer stacks with an fp32 residual stream, recurrent mixers and windowed attention over a RAGGED
+ * step (csrc/linear_any.hip, stream_ops.hip, seq_mix.hip).  No counterpart in the reference, whose
+ * only model family is the Llama-shaped one.
+ *
+ * A step's tokens lie back to back; row b (one sequence) owns tokens [row_start[b], row_start[b] +
+ * row_len[b]) and had row_ctx[b] tokens before the step; tok_row[t] / tok_pos[t] give every token's
+ * row and position.  Recurrent state lives in slot row_slot[b] of fp32 pools and is taken as zero
+ * when row_ctx[b] == 0; keys and values live in pages named by block_table[b, pos / page].
+ * `f32` selects the activation type of projection operands and cached keys/values: 0 = bf16,
+ * 1 = fp32 (the whole model in 32 bits).  Everything else is fp32 in both.
+ * ------------------------------------------------------------------------------------------------ */
+
+/* y[M,N] (fp32) = x[M,K] . W[N,K]^T, row-major operands of the activation type, any M, N, K. */
+int mv_linear_any(const void* x, int64_t ldx, const void* w, int64_t ldw, float* y, int64_t ldy, int m, int n,
+                  int k, int f32, mv_stream_t stream);
+
+/* x[r,:] = table[ids[r],:] * scale (fp32), h = the same in the activation type. */
+int mv_embed_scaled(const void* table, const int32_t* ids, float* x, int64_t ldx, void* h, int64_t ldh, int rows,
+                    int n, int vocab, float scale, int f32, mv_stream_t stream);
+
+/* v = s1*y1 (+ s2*y2 when y2 != NULL); x += v / sqrt(mean(v^2) + eps) * (1 + w); h = act(x). */
+int mv_postnorm_residual(const float* y1, int64_t ld1, const float* y2, int64_t ld2, float s1, float s2,
+                         const float* w, float eps, float* x, int64_t ldx, void* h, int64_t ldh, int rows, int n,
+                         int f32, mv_stream_t stream);
+
+/* out[r,:] = act( x[idx[r],:] / sqrt(mean(.^2) + eps) * (1 + w) ); idx == NULL: row r itself. */
+int mv_offset_rmsnorm_gather(const float* x, int64_t ldx, const int32_t* idx, const float* w, float eps, void* out,
+                             int64_t ldo, int rows, int n, int f32, mv_stream_t stream);
+
+/* out = act( max(in, 0)^2 ). */
+int mv_relu_squared(const float* in, int64_t ldi, void* out, int64_t ldo, int rows, int n, int f32,
+                    mv_stream_t stream);
+
+/* v = cap * tanh(v / cap), in place. */
+int mv_softcap(float* v, int64_t count, float cap, mv_stream_t stream);
+
+/* out[t,c] = silu(bias[c] + sum_j w[c,j] * in[t - (taps-1) + j, c]) within each row, the inputs before
+ * the row's first token taken from state[slot][taps-1][channels] (zeros for a new sequence); then the
+ * state receives the row's last taps-1 inputs.  w: fp32 [channels, taps], last column = current token. */
+int mv_conv_silu(const float* in, int64_t ldi, float* state, const float* w, const float* bias, float* out,
+                 int64_t ldo, const int32_t* tok_row, const int32_t* row_start, const int32_t* row_len,
+                 const int32_t* row_ctx, const int32_t* row_slot, int tokens, int rows, int channels, int taps,
+                 mv_stream_t stream);
+
+/* gain[t,h] = log(1 + exp(raw[t,h] + dt_bias[h])); decay[t,h] = exp(-exp(a_log[h]) * gain[t,h]). */
+int mv_softplus_decay(const float* raw, int64_t ld, const float* dt_bias, const float* a_log, float* gain,
+                      float* decay, int tokens, int heads, mv_stream_t stream);
+
+/* Per row and head, token by token: S = decay[t,h] * S + gain[t,h] * k_t v_t^T (S: n x p, fp32, in
+ * state[slot][head]); out[t, h*p ..] = S^T q_t (+ skip[h] * v_t).  q and k of head h are read at
+ * column (h / q_div) * n and (h / k_div) * n (heads that share a group); gain == NULL: 1;
+ * ld_decay == 0: decay[h] for every token. */
+int mv_scan_outer(const float* q, int64_t ldq, int q_div, const float* k, int64_t ldk, int k_div, const float* v,
+                  int64_t ldv, const float* decay, int64_t ld_decay, const float* gain, int64_t ld_gain,
+                  const float* skip, float* state, float* out, int64_t ldo, const int32_t* row_start,
+                  const int32_t* row_len, const int32_t* row_ctx, const int32_t* row_slot, int rows, int heads, int n,
+                  int p, mv_stream_t stream);
+
+/* In place, per token and head of width dim: (u, v) = (x[i], x[i + rot/2]), i < rot/2, becomes
+ * (u cos a - v sin a, v cos a + u sin a), a = tok_pos[t] * inv_freq[i] (formed in fp64); all dim values
+ * are then multiplied by scale. */
+int mv_rotary_pairs(float* x, int64_t ld, const double* inv_freq, const int32_t* tok_pos, int tokens, int heads,
+                    int dim, int rot, float scale, mv_stream_t stream);
+
+/* Rows cut into `groups` equal parts, each divided by its root mean square; gate_first: the part is
+ * y * silu(gate) before that, else silu(gate) multiplies after; w (fp32 [n]) multiplies last or is NULL. */
+int mv_gated_group_norm(const float* y, int64_t ldy, const float* gate, int64_t ldg, const float* w, void* out,
+                        int64_t ldo, int rows, int n, int groups, int gate_first, float eps, int f32,
+                        mv_stream_t stream);
+
+/* Rows of qkv are [heads x d | kv_heads x d | kv_heads x dv] fp32.  Queries are divided by their root
+ * mean square in place; keys likewise and written, with the values, to k_cache [pages, page, kv_heads, d]
+ * and v_cache [pages, page, kv_heads, dv] at the token's position. */
+int mv_qk_unitnorm_store(float* qkv, int64_t ld, void* k_cache, void* v_cache, const int32_t* tok_row,
+                         const int32_t* tok_pos, const int32_t* block_table, int bt_stride, int page, int tokens,
+                         int heads, int kv_heads, int d, int dv, float eps, int f32, mv_stream_t stream);
+
+/* out[t, h*dv ..] = softmax_j( q_t . k_j * scale - slopes[h] * (pos - j) ) v_j over pos - window < j <= pos
+ * from the pages (the step's own keys must already be stored).  dv <= 256. */
+int mv_window_attn(const float* q, int64_t ldq, const void* k_cache, const void* v_cache, void* out, int64_t ldo,
+                   const int32_t* tok_row, const int32_t* tok_pos, const int32_t* block_table, int bt_stride,
+                   int page, const float* slopes, int tokens, int heads, int kv_heads, int d, int dv, float scale,
+                   int window, int f32, mv_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -91,6 +91,20 @@ PROTOTYPES = {
     "mv_allgather_init": (_I, [_I, _I, _I, _I, ctypes.POINTER(c_void_p)]),
     "mv_allgather_rows": (_I, [_P, _P, _L, _P, _L, _I, _I, _P]),
     "mv_allreduce_addnorm": (_I, [_P, _P, _L, _P, _I, _P, _L, _P, _L, _P, _F, _P, _L, _I, _I, _I, _P]),
+    "mv_linear_any": (_I, [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _P]),
+    "mv_embed_scaled": (_I, [_P, _P, _P, _L, _P, _L, _I, _I, _I, _F, _I, _P]),
+    "mv_postnorm_residual": (_I, [_P, _L, _P, _L, _F, _F, _P, _F, _P, _L, _P, _L, _I, _I, _I, _P]),
+    "mv_offset_rmsnorm_gather": (_I, [_P, _L, _P, _P, _F, _P, _L, _I, _I, _I, _P]),
+    "mv_relu_squared": (_I, [_P, _L, _P, _L, _I, _I, _I, _P]),
+    "mv_softcap": (_I, [_P, _L, _F, _P]),
+    "mv_conv_silu": (_I, [_P, _L, _P, _P, _P, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "mv_softplus_decay": (_I, [_P, _L, _P, _P, _P, _P, _I, _I, _P]),
+    "mv_scan_outer": (_I, [_P, _L, _I, _P, _L, _I, _P, _L, _P, _L, _P, _L, _P, _P, _P, _L, _P, _P, _P, _P,
+                           _I, _I, _I, _I, _P]),
+    "mv_rotary_pairs": (_I, [_P, _L, _P, _P, _I, _I, _I, _I, _F, _P]),
+    "mv_gated_group_norm": (_I, [_P, _L, _P, _L, _P, _P, _L, _I, _I, _I, _I, _F, _I, _P]),
+    "mv_qk_unitnorm_store": (_I, [_P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P]),
+    "mv_window_attn": (_I, [_P, _L, _P, _P, _P, _L, _P, _P, _P, _I, _I, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P]),
     "mv_graph_begin_capture": (_I, [_P]),
     "mv_graph_end_capture": (_I, [_P, ctypes.POINTER(c_void_p)]),
     "mv_graph_launch": (_I, [_P, _P]),
@@ -108,16 +122,31 @@ class NativeError(RuntimeError):
         super().__init__(f"{fn} failed: status {status} ({detail})")
 
 
+def _part_libraries():
+    d = os.path.join(_HERE, "lib")
+    if not os.path.isdir(d):
+        return []
+    return sorted(os.path.join(d, f) for f in os.listdir(d) if f.startswith("libmvllm_") and f.endswith(".so"))
+
+
 def lib():
-    """Load libmvllm.so once; raise (never fall back) when it is absent."""
+    """Load libmvllm.so once; raise (never fall back to another compute path) when it is absent.  When
+    only a library of a part of the sources has been built (build.py SETS), that one is loaded and
+    the entry points it lacks raise AttributeError when they are first asked for."""
     global _lib
     if _lib is None:
-        if not os.path.exists(LIB_PATH):
-            raise ImportError(
-                f"{LIB_PATH} is missing: build it with `python micro-vllm_amd/build.py` "
-                "(hipcc --offload-arch=gfx950). There is no fallback path.")
-        handle = ctypes.CDLL(LIB_PATH)
+        path, whole = LIB_PATH, True
+        if not os.path.exists(path):
+            parts = [] if os.environ.get("MVLLM_LIB") else _part_libraries()
+            if not parts:
+                raise ImportError(
+                    f"{LIB_PATH} is missing: build it with `python micro-vllm_amd/build.py` "
+                    "(hipcc --offload-arch=gfx950). There is no fallback path.")
+            path, whole = parts[0], False
+        handle = ctypes.CDLL(path)
         for name, (res, args) in PROTOTYPES.items():
+            if not whole and not hasattr(handle, name):
+                continue
             fn = getattr(handle, name)  # AttributeError if the symbol is not exported
             fn.restype = res
             fn.argtypes = args

@@ -26,7 +26,20 @@ SOURCES = [
     "sampler.hip",
     "allreduce.hip",
     "qkv_attn.hip",
+    "linear_any.hip",
+    "stream_ops.hip",
+    "seq_mix.hip",
 ]
+
+# Libraries that hold a part of the sources, `lib/libmvllm_<name>.so`: what one model family needs, for a
+# first start in a fresh checkout that should not wait for kernels it will never launch.  The binding
+# loads such a library when the full one has not been built and resolves the entry points it finds.
+SETS = {
+    # fp32 residual stream, recurrent mixers, windowed attention; the wave-tile projections for the
+    # shapes they take, and the sampler
+    "ragged": ["runtime.hip", "linear_any.hip", "stream_ops.hip", "seq_mix.hip", "wgemm.hip",
+               "gemm_prefill.hip", "sampler.hip"],
+}
 
 # -ffp-contract=off: rounding is part of the parity contract; FMAs are written explicitly
 FLAGS = [
@@ -38,6 +51,8 @@ FLAGS = [
     "-fno-gpu-rdc",
     "-Wall",
     "-Wno-unused-function",
+    # no packed fp32 arithmetic (v_pk_*_f32): the scalar forms only
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 
 
@@ -93,13 +108,19 @@ def build_variant(name, defines, only=("wgemm.hip",), verbose=False):
     return out
 
 
-def build(force=False, verbose=True, jobs=None):
+def set_path(name):
+    return os.path.join(LIBDIR, f"libmvllm_{name}.so")
+
+
+def build(force=False, verbose=True, jobs=None, only=None):
+    """The full library, or with `only` = a key of SETS the library of that part of the sources."""
     os.makedirs(LIBDIR, exist_ok=True)
     os.makedirs(OBJDIR, exist_ok=True)
     hipcc = _hipcc()
     headers = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
     headers.append(os.path.join(HERE, "..", "include", "mvllm.h"))
-    srcs = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    srcs = [s for s in (SOURCES if only is None else SETS[only]) if os.path.exists(os.path.join(CSRC, s))]
+    LIB = globals()["LIB"] if only is None else set_path(only)
     objs = []
     todo = []
     for s in srcs:
@@ -135,5 +156,5 @@ def build(force=False, verbose=True, jobs=None):
 
 
 if __name__ == "__main__":
-    build(force="--force" in sys.argv)
-    print(LIB)
+    part = next((a.split("=", 1)[1] for a in sys.argv if a.startswith("--only=")), None)
+    print(build(force="--force" in sys.argv, only=part))

@@ -19,7 +19,8 @@ from .layer.model_prefill import ModelPrefillRunner
 from .layer.sampler import Sampler, greedy
 from .parallel_config import get_rank, get_world_size, rank0, setup
 from .scheduler import Scheduler
-from .sequence import Sequence
+from .sequence import IdTokenizer, Sequence
+from ..models.registry import family_of
 
 logger = logging.getLogger("InferenceEngine")
 
@@ -50,7 +51,8 @@ class InferenceEngine:
                  n_blocks: Optional[int] = None, max_tokens: int = 1024,
                  graph_batch_sizes: Optional[List[int]] = None, prefill_timeout: float = 0.02,
                  exact_rope: bool = False, trust_remote_code: bool = False, kv_fraction: float = 0.9,
-                 clear_unwritten_slot: bool = True, sample_last_real_token: bool = False):
+                 clear_unwritten_slot: bool = True, sample_last_real_token: bool = False,
+                 dtype: torch.dtype = torch.bfloat16, state_slots: Optional[int] = None):
         """`max_tokens` is the longest sequence a block-table row can describe (the reference's
         KVCacheManager default, 1024, gives four columns - pass more for long contexts).
         `n_blocks`: None = the reference's 81 pages (core/engine.py:53-57), a number, or "auto" =
@@ -68,7 +70,10 @@ class InferenceEngine:
         leaves the slot as it is.
         `sample_last_real_token`: take the first generated token of a right-padded prompt from the
         logits of its last REAL token instead of the batch's last (pad) position, which is what the
-        reference samples from (core/engine.py:233 with core/scheduler.py:157-163)."""
+        reference samples from (core/engine.py:233 with core/scheduler.py:157-163).
+        `dtype` / `state_slots`: for the "ragged" model family (models/registry.py), whose runner also
+        works in fp32 throughout and keeps recurrent state in `state_slots` slots (default
+        max_batch_size) beside pages of 64 tokens; `n_blocks` then counts those pages."""
         setup()
         self.rank = get_rank()
         if model is None:
@@ -85,6 +90,12 @@ class InferenceEngine:
         self.device, self.dtype = "cuda", torch.bfloat16
         self.model, self.tokenizer = model, tokenizer
         self.config = model.config
+        self.family = family_of(model)
+        if self.family == "ragged":
+            self._init_ragged(max_batch_size, max_prefill_tokens, n_blocks, max_tokens, prefill_timeout,
+                              kv_fraction, dtype, state_slots)
+            return
+        assert dtype == torch.bfloat16, "the Llama-shaped runners compute in bf16 storage / fp32 accumulate"
 
         # per-rank geometry (core/engine.py:101-114)
         cfg = self.config
@@ -138,6 +149,86 @@ class InferenceEngine:
         self.scheduler.batch_sizes = [b for b in sizes if b <= max_batch_size] or [max_batch_size]
         self.graph_runner.capture(self.cache_manager, batch_sizes=self.scheduler.batch_sizes)
 
+    # ------------------------------------------------------------------ ragged family
+    def _init_ragged(self, max_batch_size, max_prefill_tokens, n_blocks, max_tokens, prefill_timeout,
+                     kv_fraction, dtype, state_slots):
+        """Runner, cache manager and scheduler of a model whose step function takes rows of any
+        length (core/layer/ragged_runner.py): one kind of step, no graphs, no padding."""
+        from .layer.ragged_runner import RaggedRunner
+        assert get_world_size() == 1, "the ragged family runs on one rank"
+        self.dtype = dtype
+        if self.tokenizer is None:
+            self.tokenizer = IdTokenizer(self.config.vocab_size)
+        self.num_layers = self.config.num_hidden_layers
+        self.runner = RaggedRunner(self.model, self.device, dtype)
+        page = self.runner.PAGE
+        kv, _ = self.runner.cache_layout()
+        if n_blocks == "auto":
+            torch.cuda.synchronize()
+            free, _ = torch.cuda.mem_get_info()
+            per_page = sum(page * g * (d + dv) for g, d, dv in kv.values()) * (4 if dtype == torch.float32 else 2)
+            n_blocks = max(16, int(free * kv_fraction) // max(per_page, 1))
+        elif n_blocks is None:
+            n_blocks = self.DEFAULT_MAX_BLOCKS * self.DEFAULT_BLOCK_SIZE // page
+        self.cache_manager = self.runner.make_cache(
+            n_blocks, state_slots or max_batch_size, max_tokens=max_tokens, max_rows=max_batch_size,
+            max_step_tokens=max_prefill_tokens + max_batch_size)
+        self.scheduler = Scheduler(max_batch_size, max_prefill_tokens, self.tokenizer, prefill_timeout, ragged=True,
+                                   reserve=self._reserve_for)
+        self.sampler = Sampler()
+        self.eos_token_id = getattr(self.tokenizer, "eos_token_id", None)
+        self.stream_callbacks = {}
+        self.max_position = max_tokens
+
+    def _reserve_for(self, seq: Sequence, n: int) -> bool:
+        from .state_cache import PoolExhausted
+        try:
+            self.cache_manager.reserve([(seq.seq_id, n)])
+            return True
+        except PoolExhausted:
+            return False
+
+    @torch.inference_mode()
+    def run_ragged(self, entries, residuals=None) -> torch.Tensor:
+        """One step of the ragged family: entries = [(seq_id, its next token ids, wanted)], `wanted` =
+        indices into those tokens whose logits are returned (fp32 [sum of wanted, vocab], in entry
+        order).  A sequence is admitted at its first entry; what it holds stays until `release`."""
+        rows = [(sid, len(toks)) for sid, toks, _ in entries]
+        self.cache_manager.reserve(rows)
+        step = self.cache_manager.plan([(sid, toks) for sid, toks, _ in entries])
+        want, start = [], 0
+        for _, toks, wanted in entries:
+            want += [start + int(i) for i in wanted]
+            start += len(toks)
+        want_t = torch.tensor(want, dtype=torch.int32).to(self.device, non_blocking=True) if want else \
+            torch.zeros(0, dtype=torch.int32, device=self.device)
+        logits = self.runner.forward(step, self.cache_manager, want_t, residuals=residuals)
+        self.cache_manager.advance(rows)
+        return logits
+
+    def release(self, seq_id):
+        """Give back the pages and the state slot of a sequence."""
+        self.cache_manager.free(seq_id)
+
+    def _step_mixed(self, batch: List[Sequence]):
+        entries, sampling = [], []
+        for seq in batch:
+            lo, n = seq.num_computed, seq._portion
+            last = lo + n == len(seq.full_ids)
+            entries.append((seq.seq_id, seq.full_ids[lo:lo + n], [n - 1] if last else []))
+            seq._next_token = None
+            if last:
+                sampling.append(seq)
+        logits = self.run_ragged(entries)
+        for seq in batch:
+            seq.num_computed += seq._portion
+        if sampling:
+            temps = torch.tensor([max(float(s.temperature), 0.0) for s in sampling], device=self.device)
+            topp = torch.tensor([float(s.top_p) for s in sampling], device=self.device)
+            picked = self._sample(logits.to(torch.bfloat16), temps, topp, 50)
+            for seq, tok in zip(sampling, picked):
+                seq._next_token = tok
+
     def auto_kv_blocks(self, fraction: float) -> int:
         """Pages of DEFAULT_BLOCK_SIZE tokens (K and V, all layers, this rank's kv heads) that fit
         into `fraction` of the currently free device memory; never fewer than the reference's pool."""
@@ -170,6 +261,13 @@ class InferenceEngine:
         # block-table column, can never be served; the reference fails on it later, inside the
         # scheduler (TypeError) or the cache manager.  Refused here, with the limits named.
         n = len(seq.input_ids)
+        if self.family == "ragged":
+            rows = self.cache_manager.max_seq_pages * self.cache_manager.page_size
+            if n == 0 or n + max_tokens > rows:
+                raise ValueError(f"prompt of {n} tokens with max_tokens={max_tokens} cannot be scheduled: "
+                                 f"a block-table row covers {rows} positions")
+            self.scheduler.add_request(seq)
+            return seq_id
         rows = self.cache_manager.max_seq_blocks * self.cache_manager.block_size
         if n == 0 or n > self.scheduler.max_prefill_tokens or n + max_tokens + 1 > rows:
             raise ValueError(
@@ -191,7 +289,9 @@ class InferenceEngine:
     def step(self, ctx: BatchInferenceContext) -> bool:
         if not ctx.sequences:
             return False
-        if ctx.batch_type == "prefill":
+        if ctx.batch_type == "mixed":
+            self._step_mixed(ctx.sequences)
+        elif ctx.batch_type == "prefill":
             self._prefill(ctx.sequences)
         else:
             self._decode(ctx.sequences)

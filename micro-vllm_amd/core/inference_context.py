@@ -20,7 +20,7 @@ import torch.distributed as dist
 from .parallel_config import get_rank, get_world_size, rank0
 from .sequence import Sequence
 
-_TYPES = ["waiting", "prefill", "decode", "idle"]
+_TYPES = ["waiting", "prefill", "decode", "idle", "mixed"]
 _STATES = ["prefill", "decode", "finished"]
 _NONE = -(1 << 62)
 
@@ -66,7 +66,7 @@ def unpack_sequences(words: List[int], count: int, tokenizer) -> List[Sequence]:
 @dataclass
 class BatchInferenceContext:
     batch_size: int
-    batch_type: str  # "waiting" / "prefill" / "decode"
+    batch_type: str  # "waiting" / "prefill" / "decode" / "mixed" (ragged steps, one rank only)
     sequences: List[Sequence] = field(default_factory=list)
     _device: torch.device = None
 

@@ -74,10 +74,11 @@ class CheckpointFiles:
         return self._where.keys()
 
     def get(self, name: str, dtype=torch.bfloat16) -> torch.Tensor:
+        """`dtype=None`: as stored."""
         if name not in self._where:
             raise KeyError(f"tensor {name!r} is not in the checkpoint at {self.path!r}")
         t = self._file(self._where[name]).get_tensor(name)
-        return t if t.dtype == dtype else t.to(dtype)
+        return t if dtype is None or t.dtype == dtype else t.to(dtype)
 
 
 class LazyParam:
@@ -181,6 +182,13 @@ def load_weights(model_path: str) -> SyntheticModel:
     """The model object alone (no tokenizer)."""
     with open(os.path.join(model_path, "config.json")) as f:
         hf = json.load(f)
+    from ..models.registry import loader_for
+    by_architecture = loader_for(hf)
+    if by_architecture is not None:
+        model = by_architecture(hf, CheckpointFiles(model_path), os.path.basename(os.path.normpath(model_path)))
+        logger.info("checkpoint %s: architecture %s, %d layers", model_path, hf["architecture"],
+                    model.config.num_hidden_layers)
+        return model
     cfg = _config_from_hf(hf, os.path.basename(os.path.normpath(model_path)))
     files = CheckpointFiles(model_path)
     eps = cfg.layer_norm_epsilon
@@ -221,5 +229,14 @@ def load_model(model_path: str, device=None, *, tokenizer: bool = True, trust_re
     """-> (model, tokenizer).  `device` is accepted for the reference's signature; parameters stay
     in the memory-mapped files until a runner's `prepare_weights` moves this rank's shard."""
     model = load_weights(model_path)
-    tok = load_tokenizer(model_path, trust_remote_code) if tokenizer else None
+    tok = None
+    if tokenizer:
+        has_tok = any(os.path.exists(os.path.join(model_path, f))
+                      for f in ("tokenizer.json", "tokenizer.model", "tokenizer_config.json", "vocab.json"))
+        if has_tok or getattr(model, "family", "llama") == "llama":
+            tok = load_tokenizer(model_path, trust_remote_code)
+        else:
+            # a checkpoint without tokenizer files: requests are token ids written as numbers
+            from .sequence import IdTokenizer
+            tok = IdTokenizer(model.config.vocab_size)
     return model, tok

@@ -20,7 +20,9 @@ logger = logging.getLogger(__name__)
 
 class Scheduler:
     def __init__(self, max_batch_size: int = 32, max_prefill_tokens: int = 2048, tokenizer=None,
-                 prefill_timeout: float = 0.02, clock: Callable[[], float] = None):
+                 prefill_timeout: float = 0.02, clock: Callable[[], float] = None, ragged: bool = False,
+                 reserve: Callable = None):
+        self.ragged, self.reserve = ragged, reserve
         self.tokenizer = tokenizer
         self.max_batch_size = max_batch_size
         self.max_prefill_tokens = max_prefill_tokens
@@ -40,11 +42,43 @@ class Scheduler:
 
     def get_next_batch(self) -> Tuple[List[Sequence], str]:
         self.running_sequences = [s for s in self.running_sequences if not s.is_finished()]
+        if self.ragged:
+            return self._get_mixed_batch()
         if self.waiting_queue:
             batch, kind = self._get_prefill_batch()
             if kind != "idle":
                 return batch, kind           # "prefill", or "waiting" (let the caller yield)
         return self._get_decode_batch()
+
+    def _get_mixed_batch(self) -> Tuple[List[Sequence], str]:
+        rows, budget = [], self.max_prefill_tokens
+
+        def take(seq, n):
+            if self.reserve is not None and not self.reserve(seq, n):
+                return False
+            seq._portion = n
+            rows.append(seq)
+            return True
+
+        for seq in self.running_sequences:
+            if len(rows) >= self.max_batch_size or budget <= 0:
+                break
+            if seq.state == "decode" and take(seq, 1):
+                budget -= 1
+        under_way = [s for s in self.running_sequences if s.state == "prefill"]
+        for seq in under_way + list(self.waiting_queue):
+            if len(rows) >= self.max_batch_size or budget <= 0:
+                break
+            n = min(len(seq.full_ids) - seq.num_computed, budget)
+            if n <= 0 or not take(seq, n):
+                break      # arrival order is kept: nobody overtakes a prompt that has to wait
+            budget -= n
+            if seq not in self.running_sequences:
+                self.waiting_queue.remove(seq)
+                self.running_sequences.append(seq)
+        if rows:
+            return rows, "mixed"
+        return [], ("waiting" if self.waiting_queue or self.running_sequences else "idle")
 
     def _get_decode_batch(self) -> Tuple[List[Sequence], str]:
         by_position = defaultdict(list)

@@ -5,9 +5,31 @@ import time
 from typing import List, Optional
 
 
+class IdTokenizer:
+    """For checkpoints that ship no tokenizer: a prompt is its token ids written as numbers
+    ("17 4 250"), and text out is the same."""
+    eos_token_id = None
+
+    def __init__(self, vocab_size: int):
+        self.vocab_size = vocab_size
+
+    def encode(self, text, add_special_tokens=True):
+        ids = [int(t) for t in str(text).replace(",", " ").split()]
+        if any(i < 0 or i >= self.vocab_size for i in ids):
+            raise ValueError(f"token id outside [0, {self.vocab_size})")
+        return ids
+
+    def decode(self, ids, skip_special_tokens=True):
+        return " ".join(str(int(i)) for i in ids)
+
+
 class Sequence:
     # result of the last step, kept on every rank until update_state consumes it
     _next_token: Optional[int] = None
+    # ragged steps (prompts run in portions): tokens of full_ids already through the model, and how
+    # many the scheduler gave this sequence in the step under way
+    num_computed: int = 0
+    _portion: int = 0
 
     def __init__(self, seq_id: int, prompt: str, tokenizer, max_tokens: int = 128):
         self.seq_id = seq_id

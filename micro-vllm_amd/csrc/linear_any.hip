@@ -1,0 +1,139 @@
+// y[M,N] (fp32) = x[M,K] . W[N,K]^T for ANY M, N, K, row-major operands as a checkpoint stores them.
+//
+// The wave-tile projections (wgemm.hip, gemm_prefill.hip) want N % 16 == 0, K % 32 / 64 == 0 and a
+// relaid-out weight image; layer stacks whose widths are whatever their configuration says (an
+// input projection of 2*inner + 2*groups*state + heads rows, an inner width of heads * vdim) use
+// this kernel for the shapes those cannot take.  Two forms:
+//   bf16 operands: 64 x 64 output tile per workgroup of 4 waves, k in steps of 32 through LDS,
+//                  v_mfma_f32_16x16x32_bf16, edges zero-filled in LDS;
+//   fp32 operands: the same tile with fused multiply-adds (no reduced-precision matrix mode).
+// Every output is the sum over k in ascending order of 32-wide (bf16) or 16-wide (fp32) steps,
+// whatever M is: a row's result does not depend on which other rows share the launch.
+#include "common.h"
+
+namespace mv {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 la_bf16x8_t;
+
+constexpr int kLaBM = 64, kLaBN = 64, kLaBK = 32, kLaPad = 40;  // LDS row = 40 bf16 = 80 bytes
+
+__device__ __forceinline__ uint4 la_load8(const uint16_t* base, int64_t ld, int row, int nrows, int col, int k,
+                                          bool vec) {
+    if (row >= nrows || col >= k) return make_uint4(0, 0, 0, 0);
+    const uint16_t* p = base + (int64_t)row * ld + col;
+    if (vec && col + 8 <= k) return ld16(p);
+    uint16_t e[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) e[i] = (col + i < k) ? p[i] : (uint16_t)0;
+    return make_uint4(e[0] | ((uint32_t)e[1] << 16), e[2] | ((uint32_t)e[3] << 16), e[4] | ((uint32_t)e[5] << 16),
+                      e[6] | ((uint32_t)e[7] << 16));
+}
+
+__global__ __launch_bounds__(256) void linear_any_bf16_kernel(
+    const uint16_t* __restrict__ x, int64_t ldx, const uint16_t* __restrict__ w, int64_t ldw,
+    float* __restrict__ y, int64_t ldy, int M, int N, int K, int vec_x, int vec_w) {
+    __shared__ __attribute__((aligned(16))) uint16_t xs[kLaBM][kLaPad];
+    __shared__ __attribute__((aligned(16))) uint16_t ws[kLaBN][kLaPad];
+    const int m0 = blockIdx.y * kLaBM, n0 = blockIdx.x * kLaBN;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, q = lane >> 4;
+    const int lrow = tid >> 2, lcol = (tid & 3) * 8;
+    f32x4_t acc[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
+    uint4 xr = la_load8(x, ldx, m0 + lrow, M, lcol, K, vec_x);
+    uint4 wr = la_load8(w, ldw, n0 + lrow, N, lcol, K, vec_w);
+    for (int k0 = 0; k0 < K; k0 += kLaBK) {
+        __syncthreads();
+        st16(&xs[lrow][lcol], xr);
+        st16(&ws[lrow][lcol], wr);
+        __syncthreads();
+        if (k0 + kLaBK < K) {
+            xr = la_load8(x, ldx, m0 + lrow, M, k0 + kLaBK + lcol, K, vec_x);
+            wr = la_load8(w, ldw, n0 + lrow, N, k0 + kLaBK + lcol, K, vec_w);
+        }
+        // first operand: 16 weight rows of this wave; second: 16 activation rows per m-tile
+        const la_bf16x8_t wf = __builtin_bit_cast(la_bf16x8_t, ld16(&ws[wave * 16 + r][q * 8]));
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) {
+            const la_bf16x8_t xf = __builtin_bit_cast(la_bf16x8_t, ld16(&xs[mt * 16 + r][q * 8]));
+            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf, acc[mt], 0, 0, 0);
+        }
+    }
+    // acc[mt][j] = C[n = n0 + 16 wave + 4 q + j][m = m0 + 16 mt + r]
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+        const int m = m0 + mt * 16 + r;
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + wave * 16 + q * 4 + j;
+            if (n < N) y[(int64_t)m * ldy + n] = acc[mt][j];
+        }
+    }
+}
+
+constexpr int kLfBK = 16;
+
+__global__ __launch_bounds__(256) void linear_any_f32_kernel(
+    const float* __restrict__ x, int64_t ldx, const float* __restrict__ w, int64_t ldw,
+    float* __restrict__ y, int64_t ldy, int M, int N, int K) {
+    __shared__ float xs[kLfBK][kLaBM + 4];
+    __shared__ float ws[kLfBK][kLaBN + 4];
+    const int m0 = blockIdx.y * kLaBM, n0 = blockIdx.x * kLaBN;
+    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    const int lrow = tid >> 2, lcol = (tid & 3) * 4;
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < K; k0 += kLfBK) {
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int kk = k0 + lcol + i;
+            xs[lcol + i][lrow] = (m0 + lrow < M && kk < K) ? x[(int64_t)(m0 + lrow) * ldx + kk] : 0.f;
+            ws[lcol + i][lrow] = (n0 + lrow < N && kk < K) ? w[(int64_t)(n0 + lrow) * ldw + kk] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < kLfBK; ++kk) {
+            float a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                a[i] = xs[kk][ty * 4 + i];
+                b[i] = ws[kk][tx * 4 + i];
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = m0 + ty * 4 + i;
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tx * 4 + j;
+            if (n < N) y[(int64_t)m * ldy + n] = acc[i][j];
+        }
+    }
+}
+
+}  // namespace mv
+
+extern "C" int mv_linear_any(const void* x, int64_t ldx, const void* w, int64_t ldw, float* y, int64_t ldy,
+                             int m, int n, int k, int f32, mv_stream_t stream) {
+    using namespace mv;
+    if (m < 0 || n <= 0 || k <= 0) return MV_ERR_INVALID_ARG;
+    if (m == 0) return MV_OK;
+    if (!x || !w || !y || ldx < k || ldw < k || ldy < n) return MV_ERR_INVALID_ARG;
+    const dim3 grid((n + kLaBN - 1) / kLaBN, (m + kLaBM - 1) / kLaBM);
+    if (grid.y > 65535) return MV_ERR_UNSUPPORTED;
+    hipStream_t s = (hipStream_t)stream;
+    if (f32) {
+        hipLaunchKernelGGL(linear_any_f32_kernel, grid, dim3(256), 0, s, (const float*)x, ldx, (const float*)w, ldw,
+                           y, ldy, m, n, k);
+    } else {
+        const int vx = aligned16(x) && ldx % 8 == 0, vw = aligned16(w) && ldw % 8 == 0;
+        hipLaunchKernelGGL(linear_any_bf16_kernel, grid, dim3(256), 0, s, (const uint16_t*)x, ldx, (const uint16_t*)w,
+                           ldw, y, ldy, m, n, k, vx, vw);
+    }
+    return check_launch();
+}

@@ -1,0 +1,436 @@
+// Token mixers over a RAGGED step: the tokens of all rows of a step lie back to back, row b owning
+// tokens [row_start[b], row_start[b] + row_len[b]) that continue its sequence at position row_ctx[b]
+// (a prompt's portion of any length beside single decoded tokens).  What a sequence carries between
+// steps lives either in pages of a key/value pool (block_table) or in its state slot (row_slot);
+// a row with row_ctx == 0 starts from zero state whatever its slot held before.
+//
+//   conv_silu / conv_state_update  short causal convolution per channel with its tail kept per slot
+//   softplus_decay                 step sizes and decays of a selective state-space head
+//   scan_outer                     S_t = decay_t S_(t-1) + gain_t k_t v_t^T,  o_t = S_t^T q_t (+ skip_h v_t)
+//                                  (state-space duality heads and fixed-decay retention heads alike)
+//   rotary_pairs                   rotate-half rotation of the first `rot` dimensions of each head
+//   gated_group_norm               unit-RMS per group with a SiLU gate before or after it
+//   qk_unitnorm_store              per-head unit-RMS of queries and keys, keys/values into their pages
+//   window_attn                    softmax attention over the last `window` positions with a per-head
+//                                  linear distance penalty
+// All of it in fp32; the activation type (bf16 or fp32) only concerns what goes to a projection or
+// into the key/value pages.
+#include "common.h"
+
+namespace mv {
+
+template <bool F32> struct ActS;
+template <> struct ActS<true> {
+    typedef float T;
+    static __device__ __forceinline__ float ld(const float* p) { return *p; }
+    static __device__ __forceinline__ void st(float* p, float v) { *p = v; }
+};
+template <> struct ActS<false> {
+    typedef uint16_t T;
+    static __device__ __forceinline__ float ld(const uint16_t* p) { return bf16_bits_to_f32(*p); }
+    static __device__ __forceinline__ void st(uint16_t* p, float v) { *p = (uint16_t)f32_to_bf16_bits(v); }
+};
+
+__device__ __forceinline__ float silu_f(float v) { return v / (1.0f + expf(-v)); }
+
+struct StepRows {
+    const int* tok_row;    // [T] row of each token
+    const int* tok_pos;    // [T] position of each token in its sequence
+    const int* row_start;  // [B]
+    const int* row_len;    // [B]
+    const int* row_ctx;    // [B] tokens the sequence held before this step
+    const int* row_slot;   // [B] state slot
+};
+
+constexpr int kMaxTaps = 16;
+
+__global__ __launch_bounds__(256) void conv_silu_kernel(const float* in, int64_t ldi, const float* state,
+                                                        const float* w, const float* bias, float* out, int64_t ldo,
+                                                        StepRows r, int T, int C, int taps) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (int64_t)T * C) return;
+    const int t = (int)(i / C), c = (int)(i % C);
+    const int b = r.tok_row[t];
+    const int rel = t - r.row_start[b];
+    const bool carried = r.row_ctx[b] > 0;
+    const float* st = state + ((int64_t)r.row_slot[b] * (taps - 1)) * C + c;
+    float acc = bias ? bias[c] : 0.f;
+    for (int j = 0; j < taps; ++j) {
+        const int src = rel - (taps - 1) + j;  // portion-relative index of the input under tap j
+        float v;
+        if (src >= 0) v = in[(int64_t)(t - (taps - 1) + j) * ldi + c];
+        else v = carried ? st[(int64_t)(src + taps - 1) * C] : 0.f;
+        acc = fmaf(w[(int64_t)c * taps + j], v, acc);
+    }
+    out[(int64_t)t * ldo + c] = silu_f(acc);
+}
+
+__global__ __launch_bounds__(256) void conv_state_update_kernel(const float* in, int64_t ldi, float* state,
+                                                                StepRows r, int B, int C, int taps) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (int64_t)B * C) return;
+    const int b = (int)(i / C), c = (int)(i % C);
+    const int keep = taps - 1, len = r.row_len[b], start = r.row_start[b];
+    const bool carried = r.row_ctx[b] > 0;
+    float* st = state + ((int64_t)r.row_slot[b] * keep) * C + c;
+    float old[kMaxTaps];
+    for (int s = 0; s < keep; ++s) old[s] = carried ? st[(int64_t)s * C] : 0.f;
+    for (int s = 0; s < keep; ++s) {
+        const int rel = len - keep + s;
+        st[(int64_t)s * C] = rel >= 0 ? in[(int64_t)(start + rel) * ldi + c] : old[s + len];
+    }
+}
+
+__global__ __launch_bounds__(256) void softplus_decay_kernel(const float* raw, int64_t ld, const float* dt_bias,
+                                                             const float* a_log, float* gain, float* decay, int T,
+                                                             int H) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= T * H) return;
+    const int t = i / H, h = i % H;
+    const float v = raw[(int64_t)t * ld + h] + dt_bias[h];
+    const float dt = fmaxf(v, 0.f) + log1pf(expf(-fabsf(v)));  // log(1 + e^v), no clamp
+    gain[i] = dt;
+    decay[i] = expf(-expf(a_log[h]) * dt);
+}
+
+struct ScanArgs {
+    const float *q, *k, *v, *decay, *gain, *skip;
+    int64_t ldq, ldk, ldv, ld_decay, ld_gain, ldo;
+    int q_div, k_div;
+    float* state;
+    float* out;
+    StepRows r;
+    int H, n, p, pt;
+};
+
+template <int MAXN>
+__global__ __launch_bounds__(256) void scan_outer_kernel(ScanArgs a) {
+    __shared__ float part[2][256];
+    const int b = blockIdx.z, h = blockIdx.y, tid = threadIdx.x;
+    const int PT = a.pt, NS = 256 / PT;
+    const int cl = tid % PT, ng = tid / PT, c = blockIdx.x * PT + cl;
+    const bool vc = c < a.p;
+    const int npt = (a.n + NS - 1) / NS, n0 = ng * npt;
+    const int len = a.r.row_len[b], start = a.r.row_start[b];
+    const bool carried = a.r.row_ctx[b] > 0;
+    float* sp = a.state + (((int64_t)a.r.row_slot[b] * a.H + h) * a.n + n0) * a.p + c;
+    float S[MAXN];
+#pragma unroll
+    for (int i = 0; i < MAXN; ++i) S[i] = (carried && vc && i < npt && n0 + i < a.n) ? sp[(int64_t)i * a.p] : 0.f;
+    for (int t = 0; t < len; ++t) {
+        const int64_t tok = start + t;
+        const float dec = a.decay[tok * a.ld_decay + h];
+        const float g = a.gain ? a.gain[tok * a.ld_gain + h] : 1.0f;
+        const float vv = vc ? a.v[tok * a.ldv + (int64_t)h * a.p + c] : 0.f;
+        const float gv = g * vv;
+        const float* kp = a.k + tok * a.ldk + (int64_t)(h / a.k_div) * a.n + n0;
+        const float* qp = a.q + tok * a.ldq + (int64_t)(h / a.q_div) * a.n + n0;
+        float o = 0.f;
+#pragma unroll
+        for (int i = 0; i < MAXN; ++i) {
+            if (i < npt && n0 + i < a.n) {
+                S[i] = fmaf(kp[i], gv, dec * S[i]);
+                o = fmaf(S[i], qp[i], o);
+            }
+        }
+        part[t & 1][tid] = o;
+        __syncthreads();
+        if (ng == 0 && vc) {
+            float tot = 0.f;
+            for (int j = 0; j < NS; ++j) tot += part[t & 1][j * PT + cl];
+            if (a.skip) tot = fmaf(a.skip[h], vv, tot);
+            a.out[tok * a.ldo + (int64_t)h * a.p + c] = tot;
+        }
+    }
+    if (vc) {
+#pragma unroll
+        for (int i = 0; i < MAXN; ++i)
+            if (i < npt && n0 + i < a.n) sp[(int64_t)i * a.p] = S[i];
+    }
+}
+
+__global__ __launch_bounds__(256) void rotary_pairs_kernel(float* x, int64_t ld, const double* inv_freq,
+                                                           const int* tok_pos, int T, int heads, int dim, int rot,
+                                                           float scale) {
+    const int half = rot / 2, per = dim - half;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (int64_t)T * heads * per) return;
+    const int j = (int)(i % per), hh = (int)((i / per) % heads), t = (int)(i / ((int64_t)per * heads));
+    float* p = x + (int64_t)t * ld + (int64_t)hh * dim;
+    if (j < half) {
+        const double ang = (double)tok_pos[t] * inv_freq[j];
+        const float cs = (float)cos(ang), sn = (float)sin(ang);
+        const float u = p[j], v = p[j + half];
+        p[j] = (u * cs - v * sn) * scale;
+        p[j + half] = (v * cs + u * sn) * scale;
+    } else {
+        p[j + half] *= scale;
+    }
+}
+
+template <bool F32>
+__global__ __launch_bounds__(256) void gated_group_norm_kernel(const float* y, int64_t ldy, const float* gate,
+                                                               int64_t ldg, const float* w, void* out_, int64_t ldo,
+                                                               int rows, int n, int groups, int gate_first,
+                                                               float eps) {
+    typedef typename ActS<F32>::T T;
+    T* out = (T*)out_;
+    const int unit = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (unit >= rows * groups) return;
+    const int row = unit / groups, g = unit % groups, gs = n / groups;
+    const float* yr = y + (int64_t)row * ldy + (int64_t)g * gs;
+    const float* gr = gate + (int64_t)row * ldg + (int64_t)g * gs;
+    float ss = 0.f;
+    for (int c = lane; c < gs; c += 64) {
+        const float u = gate_first ? yr[c] * silu_f(gr[c]) : yr[c];
+        ss += u * u;
+    }
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)gs + eps);
+    for (int c = lane; c < gs; c += 64) {
+        float u = gate_first ? (yr[c] * silu_f(gr[c])) * inv : (yr[c] * inv) * silu_f(gr[c]);
+        if (w) u *= w[g * gs + c];
+        ActS<F32>::st(out + (int64_t)row * ldo + (int64_t)g * gs + c, u);
+    }
+}
+
+struct PagedRows {
+    const int* tok_row;
+    const int* tok_pos;
+    const int* block_table;
+    int bt_stride, page;
+};
+
+template <bool F32>
+__global__ __launch_bounds__(256) void qk_unitnorm_store_kernel(float* qkv, int64_t ld, void* kc_, void* vc_,
+                                                                PagedRows pr, int T, int H, int G, int d, int dv,
+                                                                float eps) {
+    typedef typename ActS<F32>::T T_;
+    T_* kc = (T_*)kc_;
+    T_* vc = (T_*)vc_;
+    const int per = H + 2 * G;
+    const int64_t unit = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (unit >= (int64_t)T * per) return;
+    const int t = (int)(unit / per), u = (int)(unit % per);
+    float* row = qkv + (int64_t)t * ld;
+    const int pos = pr.tok_pos[t];
+    const int pg = pr.block_table[(int64_t)pr.tok_row[t] * pr.bt_stride + pos / pr.page];
+    const int64_t slot = (int64_t)pg * pr.page + pos % pr.page;
+    if (u < H + G) {
+        float* p = row + (u < H ? (int64_t)u * d : (int64_t)H * d + (int64_t)(u - H) * d);
+        float ss = 0.f;
+        for (int c = lane; c < d; c += 64) ss += p[c] * p[c];
+        ss = wave_sum(ss);
+        const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+        if (u < H) {
+            for (int c = lane; c < d; c += 64) p[c] = p[c] * inv;
+        } else if (pg >= 0) {
+            T_* dst = kc + (slot * G + (u - H)) * d;
+            for (int c = lane; c < d; c += 64) ActS<F32>::st(dst + c, p[c] * inv);
+        }
+    } else if (pg >= 0) {
+        const int g = u - H - G;
+        const float* p = row + (int64_t)(H + G) * d + (int64_t)g * dv;
+        T_* dst = vc + (slot * G + g) * dv;
+        for (int c = lane; c < dv; c += 64) ActS<F32>::st(dst + c, p[c]);
+    }
+}
+
+constexpr int kMaxVC = 4;  // value columns per lane: vdim <= 256
+
+template <bool F32>
+__global__ __launch_bounds__(256) void window_attn_kernel(const float* q, int64_t ldq, const void* kc_,
+                                                          const void* vc_, void* out_, int64_t ldo, PagedRows pr,
+                                                          const float* slopes, int T, int H, int G, int d, int dv,
+                                                          float scale, int window) {
+    typedef typename ActS<F32>::T T_;
+    extern __shared__ float lds[];
+    const T_* kc = (const T_*)kc_;
+    const T_* vc = (const T_*)vc_;
+    T_* out = (T_*)out_;
+    const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    float* qs = lds + wv * (d + 64);
+    float* ps = qs + d;
+    const int64_t unit = (int64_t)blockIdx.x * 4 + wv;
+    if (unit >= (int64_t)T * H) return;   // whole waves leave; no block-wide barrier below
+    const int t = (int)(unit / H), h = (int)(unit % H), g = h / (H / G);
+    const int pos = pr.tok_pos[t];
+    const int* bt = pr.block_table + (int64_t)pr.tok_row[t] * pr.bt_stride;
+    const int lo = pos - window + 1 > 0 ? pos - window + 1 : 0;
+    const float slope = slopes ? slopes[h] : 0.f;
+    for (int c = lane; c < d; c += 64) qs[c] = q[(int64_t)t * ldq + (int64_t)h * d + c];
+    __builtin_amdgcn_wave_barrier();   // qs and ps are exchanged between the lanes of this wave only
+    float m = -INFINITY, l = 0.f, acc[kMaxVC] = {0.f, 0.f, 0.f, 0.f};
+    for (int j0 = lo; j0 <= pos; j0 += 64) {
+        const int j = j0 + lane;
+        float s = -INFINITY;
+        if (j <= pos) {
+            const int pg = bt[j / pr.page];
+            const T_* kr = kc + (((int64_t)pg * pr.page + j % pr.page) * G + g) * d;
+            float dot = 0.f;
+            for (int c = 0; c < d; ++c) dot = fmaf(qs[c], ActS<F32>::ld(kr + c), dot);
+            s = dot * scale - slope * (float)(pos - j);
+        }
+        const float mn = fmaxf(m, wave_max(s));
+        const float p = j <= pos ? expf(s - mn) : 0.f;
+        const float corr = expf(m - mn);   // m = -inf on the first tile: exp(-inf) = 0
+        l = l * corr + wave_sum(p);
+        m = mn;
+        __builtin_amdgcn_wave_barrier();
+        ps[lane] = p;
+        __builtin_amdgcn_wave_barrier();
+        const int cnt = pos - j0 + 1 < 64 ? pos - j0 + 1 : 64;
+#pragma unroll
+        for (int ci = 0; ci < kMaxVC; ++ci) acc[ci] *= corr;
+        for (int jj = 0; jj < cnt; ++jj) {
+            const int jk = j0 + jj;
+            const int pg = bt[jk / pr.page];
+            const T_* vr = vc + (((int64_t)pg * pr.page + jk % pr.page) * G + g) * dv;
+            const float pj = ps[jj];
+#pragma unroll
+            for (int ci = 0; ci < kMaxVC; ++ci) {
+                const int c = lane + ci * 64;
+                if (c < dv) acc[ci] = fmaf(pj, ActS<F32>::ld(vr + c), acc[ci]);
+            }
+        }
+    }
+#pragma unroll
+    for (int ci = 0; ci < kMaxVC; ++ci) {
+        const int c = lane + ci * 64;
+        if (c < dv) ActS<F32>::st(out + (int64_t)t * ldo + (int64_t)h * dv + c, acc[ci] / l);
+    }
+}
+
+}  // namespace mv
+
+extern "C" {
+
+using mv::StepRows;
+
+int mv_conv_silu(const float* in, int64_t ldi, float* state, const float* w, const float* bias, float* out,
+                 int64_t ldo, const int32_t* tok_row, const int32_t* row_start, const int32_t* row_len,
+                 const int32_t* row_ctx, const int32_t* row_slot, int tokens, int rows, int channels, int taps,
+                 mv_stream_t stream) {
+    using namespace mv;
+    if (tokens < 0 || rows < 0 || channels <= 0 || taps < 1 || taps > kMaxTaps) return MV_ERR_INVALID_ARG;
+    if (tokens == 0) return MV_OK;
+    if (!in || !state || !w || !out || ldi < channels || ldo < channels) return MV_ERR_INVALID_ARG;
+    StepRows r{tok_row, nullptr, row_start, row_len, row_ctx, row_slot};
+    hipStream_t s = (hipStream_t)stream;
+    const int64_t work = (int64_t)tokens * channels;
+    hipLaunchKernelGGL(conv_silu_kernel, dim3((unsigned)((work + 255) / 256)), dim3(256), 0, s, in, ldi, state, w, bias,
+                       out, ldo, r, tokens, channels, taps);
+    if (taps > 1) {
+        const int64_t w2 = (int64_t)rows * channels;
+        hipLaunchKernelGGL(conv_state_update_kernel, dim3((unsigned)((w2 + 255) / 256)), dim3(256), 0, s, in, ldi, state,
+                           r, rows, channels, taps);
+    }
+    return check_launch();
+}
+
+int mv_softplus_decay(const float* raw, int64_t ld, const float* dt_bias, const float* a_log, float* gain,
+                      float* decay, int tokens, int heads, mv_stream_t stream) {
+    using namespace mv;
+    if (tokens < 0 || heads <= 0) return MV_ERR_INVALID_ARG;
+    if (tokens == 0) return MV_OK;
+    if (!raw || !dt_bias || !a_log || !gain || !decay || ld < heads) return MV_ERR_INVALID_ARG;
+    hipLaunchKernelGGL(softplus_decay_kernel, dim3((tokens * heads + 255) / 256), dim3(256), 0, (hipStream_t)stream,
+                       raw, ld, dt_bias, a_log, gain, decay, tokens, heads);
+    return check_launch();
+}
+
+int mv_scan_outer(const float* q, int64_t ldq, int q_div, const float* k, int64_t ldk, int k_div, const float* v,
+                  int64_t ldv, const float* decay, int64_t ld_decay, const float* gain, int64_t ld_gain,
+                  const float* skip, float* state, float* out, int64_t ldo, const int32_t* row_start,
+                  const int32_t* row_len, const int32_t* row_ctx, const int32_t* row_slot, int rows, int heads, int n,
+                  int p, mv_stream_t stream) {
+    using namespace mv;
+    if (rows < 0 || heads <= 0 || n <= 0 || p <= 0 || q_div <= 0 || k_div <= 0) return MV_ERR_INVALID_ARG;
+    if (rows == 0) return MV_OK;
+    if (!q || !k || !v || !decay || !state || !out || rows > 65535 || heads > 65535) return MV_ERR_INVALID_ARG;
+    ScanArgs a;
+    a.q = q; a.k = k; a.v = v; a.decay = decay; a.gain = gain; a.skip = skip;
+    a.ldq = ldq; a.ldk = ldk; a.ldv = ldv; a.ld_decay = ld_decay; a.ld_gain = ld_gain; a.ldo = ldo;
+    a.q_div = q_div; a.k_div = k_div; a.state = state; a.out = out;
+    a.r = StepRows{nullptr, nullptr, row_start, row_len, row_ctx, row_slot};
+    a.H = heads; a.n = n; a.p = p;
+    a.pt = p % 64 == 0 ? 64 : (p % 32 == 0 ? 32 : 16);
+    const int ns = 256 / a.pt, npt = (n + ns - 1) / ns;
+    const dim3 grid((p + a.pt - 1) / a.pt, heads, rows);
+    hipStream_t s = (hipStream_t)stream;
+    if (npt <= 4) hipLaunchKernelGGL(scan_outer_kernel<4>, grid, dim3(256), 0, s, a);
+    else if (npt <= 16) hipLaunchKernelGGL(scan_outer_kernel<16>, grid, dim3(256), 0, s, a);
+    else if (npt <= 64) hipLaunchKernelGGL(scan_outer_kernel<64>, grid, dim3(256), 0, s, a);
+    else return MV_ERR_UNSUPPORTED;
+    return check_launch();
+}
+
+int mv_rotary_pairs(float* x, int64_t ld, const double* inv_freq, const int32_t* tok_pos, int tokens, int heads,
+                    int dim, int rot, float scale, mv_stream_t stream) {
+    using namespace mv;
+    if (tokens < 0 || heads <= 0 || dim <= 0 || rot < 0 || rot > dim || rot % 2) return MV_ERR_INVALID_ARG;
+    if (tokens == 0) return MV_OK;
+    if (!x || !tok_pos || (rot > 0 && !inv_freq) || ld < (int64_t)heads * dim) return MV_ERR_INVALID_ARG;
+    const int64_t work = (int64_t)tokens * heads * (dim - rot / 2);
+    hipLaunchKernelGGL(rotary_pairs_kernel, dim3((unsigned)((work + 255) / 256)), dim3(256), 0, (hipStream_t)stream, x,
+                       ld, inv_freq, tok_pos, tokens, heads, dim, rot, scale);
+    return check_launch();
+}
+
+int mv_gated_group_norm(const float* y, int64_t ldy, const float* gate, int64_t ldg, const float* w, void* out,
+                        int64_t ldo, int rows, int n, int groups, int gate_first, float eps, int f32,
+                        mv_stream_t stream) {
+    using namespace mv;
+    if (rows < 0 || n <= 0 || groups <= 0 || n % groups) return MV_ERR_INVALID_ARG;
+    if (rows == 0) return MV_OK;
+    if (!y || !gate || !out || ldy < n || ldg < n || ldo < n) return MV_ERR_INVALID_ARG;
+    const int64_t units = (int64_t)rows * groups;
+    const dim3 grid((unsigned)((units + 3) / 4));
+    hipStream_t s = (hipStream_t)stream;
+    if (f32) hipLaunchKernelGGL(gated_group_norm_kernel<true>, grid, dim3(256), 0, s, y, ldy, gate, ldg, w, out, ldo, rows, n, groups, gate_first, eps);
+    else hipLaunchKernelGGL(gated_group_norm_kernel<false>, grid, dim3(256), 0, s, y, ldy, gate, ldg, w, out, ldo, rows, n, groups, gate_first, eps);
+    return check_launch();
+}
+
+int mv_qk_unitnorm_store(float* qkv, int64_t ld, void* k_cache, void* v_cache, const int32_t* tok_row,
+                         const int32_t* tok_pos, const int32_t* block_table, int bt_stride, int page, int tokens,
+                         int heads, int kv_heads, int d, int dv, float eps, int f32, mv_stream_t stream) {
+    using namespace mv;
+    if (tokens < 0 || heads <= 0 || kv_heads <= 0 || d <= 0 || dv <= 0 || page <= 0 || heads % kv_heads)
+        return MV_ERR_INVALID_ARG;
+    if (tokens == 0) return MV_OK;
+    if (!qkv || !k_cache || !v_cache || !tok_row || !tok_pos || !block_table ||
+        ld < (int64_t)(heads + kv_heads) * d + (int64_t)kv_heads * dv)
+        return MV_ERR_INVALID_ARG;
+    PagedRows pr{tok_row, tok_pos, block_table, bt_stride, page};
+    const int64_t units = (int64_t)tokens * (heads + 2 * kv_heads);
+    const dim3 grid((unsigned)((units + 3) / 4));
+    hipStream_t s = (hipStream_t)stream;
+    if (f32) hipLaunchKernelGGL(qk_unitnorm_store_kernel<true>, grid, dim3(256), 0, s, qkv, ld, k_cache, v_cache, pr, tokens, heads, kv_heads, d, dv, eps);
+    else hipLaunchKernelGGL(qk_unitnorm_store_kernel<false>, grid, dim3(256), 0, s, qkv, ld, k_cache, v_cache, pr, tokens, heads, kv_heads, d, dv, eps);
+    return check_launch();
+}
+
+int mv_window_attn(const float* q, int64_t ldq, const void* k_cache, const void* v_cache, void* out, int64_t ldo,
+                   const int32_t* tok_row, const int32_t* tok_pos, const int32_t* block_table, int bt_stride,
+                   int page, const float* slopes, int tokens, int heads, int kv_heads, int d, int dv, float scale,
+                   int window, int f32, mv_stream_t stream) {
+    using namespace mv;
+    if (tokens < 0 || heads <= 0 || kv_heads <= 0 || d <= 0 || dv <= 0 || page <= 0 || window <= 0 ||
+        heads % kv_heads)
+        return MV_ERR_INVALID_ARG;
+    if (dv > 64 * kMaxVC || d > 4096) return MV_ERR_UNSUPPORTED;
+    if (tokens == 0) return MV_OK;
+    if (!q || !k_cache || !v_cache || !out || !tok_row || !tok_pos || !block_table) return MV_ERR_INVALID_ARG;
+    PagedRows pr{tok_row, tok_pos, block_table, bt_stride, page};
+    const int64_t units = (int64_t)tokens * heads;
+    const dim3 grid((unsigned)((units + 3) / 4));
+    const size_t lds = (size_t)4 * (d + 64) * sizeof(float);
+    hipStream_t s = (hipStream_t)stream;
+    if (f32) hipLaunchKernelGGL(window_attn_kernel<true>, grid, dim3(256), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window);
+    else hipLaunchKernelGGL(window_attn_kernel<false>, grid, dim3(256), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window);
+    return check_launch();
+}
+
+}  // extern "C"
