@@ -65,6 +65,13 @@ def parse():
     ap.add_argument("--one-split-rule", action="store_true",
                     help="A/B switch: never replay the finer-split graph for rows of uneven length")
     ap.add_argument("--shapes", action="store_true", help="per-projection GB/s table on stderr")
+    ap.add_argument("--pagazen", action="store_true",
+                    help="instead of the default workload: prefill and decode throughput of the Pagazen design "
+                         "(ragged steps, recurrent mixers, windowed attention; random weights) at a few widths, "
+                         "beside the Llama-shaped model of equal width, depth and feed-forward parameters; "
+                         "one JSON line of its own")
+    ap.add_argument("--pagazen-widths", default="1024,2048,4096")
+    ap.add_argument("--pagazen-kernels", action="store_true", help="with --pagazen: per-op times of one layer pair on stderr")
     return ap.parse_args()
 
 
@@ -517,6 +524,147 @@ def cpu_baseline(args, cfg, runner, dev):
     }
 
 
+def _events_ms(fn, reps):
+    fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1) / reps
+
+
+def pagazen_compare(args, dev):
+    """Prefill (one prompt of --ctx tokens) and decode (bs 1 and 8 at context --ctx) of the Pagazen design
+    through its engine entry point (InferenceEngine.run_ragged), and the Llama-shaped runners at equal
+    width / depth / feed-forward parameters beside it.  Random weights, 4 layers per model (3 mamba2 +
+    1 parallel for Pagazen), vocabulary 32000."""
+    import micro_vllm_amd  # noqa: F401
+    from micro_vllm_amd.core.cache_manager import KVCacheManager
+    from micro_vllm_amd.core.engine import InferenceEngine
+    from micro_vllm_amd.core.layer.model_graph import ModelGraphRunner
+    from micro_vllm_amd.core.layer.model_prefill import ModelPrefillRunner
+    from micro_vllm_amd.models import SyntheticConfig, build_synthetic_model
+    from micro_vllm_amd.models.pagazen import bench_config, build_random_model
+
+    S, layers, rows = args.ctx, 4, []
+    for width in [int(w) for w in args.pagazen_widths.split(",")]:
+        row = {"width": width, "layers": layers, "ctx": S}
+        # ---- Pagazen ----
+        cfg = bench_config(width, layers)
+        eng = InferenceEngine(model=build_random_model(cfg, seed=1), max_batch_size=8, max_prefill_tokens=S,
+                              n_blocks=9 * (S // 64 + 4), max_tokens=S + 256, state_slots=9)
+        ids = torch.randint(0, cfg.vocab_size, (S,), generator=torch.Generator().manual_seed(0)).tolist()
+
+        def prefill():
+            eng.run_ragged([("p", ids, [S - 1])])
+            eng.release("p")
+        ms = _events_ms(prefill, 3)
+        row["pagazen_prefill_tok_s"] = round(S / ms * 1e3, 1)
+        for bs in (1, 8):
+            eng.run_ragged([(i, ids, []) for i in range(bs)] if bs * S <= eng.cache_manager.max_step_tokens else
+                           [(0, ids, [])])
+            if bs * S > eng.cache_manager.max_step_tokens:
+                for i in range(1, bs):
+                    eng.run_ragged([(i, ids, [])])
+            ms = _events_ms(lambda: eng.run_ragged([(i, [7], [0]) for i in range(bs)]), 20)
+            row[f"pagazen_decode_bs{bs}_tok_s"] = round(bs / ms * 1e3, 1)
+            row[f"pagazen_decode_bs{bs}_ms"] = round(ms, 3)
+            for i in range(bs):
+                eng.release(i)
+        row["pagazen_weight_GB"] = round(eng.runner.weight_bytes / 1e9, 3)
+        if args.pagazen_kernels:
+            pagazen_kernel_table(eng, ids, width)
+        del eng
+        torch.cuda.empty_cache()
+        # ---- Llama-shaped, equal width / depth; gate+up+down hold what up+down of 4 x width hold ----
+        ffn = (8 * width // 3 + 255) // 256 * 256
+        lc = SyntheticConfig(f"llama-w{width}", 32000, width, layers, width // 128, max(1, width // 512), 128, ffn, 1e-5)
+        model = build_synthetic_model(lc, dev, seed=1)
+        blocks = (S + 300) // 256 + 2
+        common = dict(model=model, num_layers=layers, num_heads=lc.num_attention_heads, head_size=128,
+                      kv_num_heads=lc.num_key_value_heads, hidden_dim=width, intermediate_size=lc.intermediate_size,
+                      device=dev, max_blocks=max(32, blocks))
+        pre = ModelPrefillRunner(max_batch_size=1, **common)
+        mgr = KVCacheManager(blocks + 1, 256, layers, lc.num_key_value_heads, 128, dtype=torch.bfloat16, device=dev,
+                             max_tokens=blocks * 256, max_batch_size=1)
+        assert mgr.alloc(0, S)[0]
+        mgr.cache_batch_data([0], [S])
+        pids = torch.tensor([ids]).to(dev)
+        ms = _events_ms(lambda: pre.forward(pids, mgr, 1, last_token_only=True), 3)
+        row["llama_prefill_tok_s"] = round(S / ms * 1e3, 1)
+        del pre, mgr
+        for bs in (1, 8):
+            dec = ModelGraphRunner(max_batch_size=bs, **common)
+            mgr = KVCacheManager(bs * blocks + 2, 256, layers, lc.num_key_value_heads, 128, dtype=torch.bfloat16,
+                                 device=dev, max_tokens=blocks * 256, max_batch_size=bs)
+            for sid in range(bs):
+                assert mgr.alloc(sid, S)[0]
+            dec.capture(mgr, batch_sizes=[bs])
+            tok = torch.zeros(bs, dtype=torch.long, device=dev)
+            pos = [S + 1]
+
+            def step():
+                for sid in range(bs):
+                    mgr.append(sid)
+                mgr.cache_batch_data(list(range(bs)), [pos[0]] * bs)
+                pos[0] += 1
+                return dec.greedy_ids(dec.forward(tok, mgr, bs))
+            ms = _events_ms(step, 20)
+            row[f"llama_decode_bs{bs}_tok_s"] = round(bs / ms * 1e3, 1)
+            row[f"llama_decode_bs{bs}_ms"] = round(ms, 3)
+            del dec, mgr
+        row["llama_weight_GB"] = round(lc.weight_bytes() / 1e9, 3)
+        del model
+        torch.cuda.empty_cache()
+        log(f"[bench] {row}")
+        rows.append(row)
+    print(json.dumps({"metric": "Pagazen beside the Llama-shaped family: prefill and decode tokens/s at equal size",
+                      "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "n_gpus": 1, "rows": rows}), flush=True)
+
+
+def pagazen_kernel_table(eng, ids, width):
+    """Per-op time of one prefill step and one single-token step (rocprof-free: HIP events around each
+    wrapper call), printed on stderr."""
+    from micro_vllm_amd.kernel import ragged_ops as ops
+    import functools
+    times = {}
+    names = ["embed_scaled", "postnorm_residual", "offset_rmsnorm_gather", "relu_squared", "softcap_", "conv_silu",
+             "softplus_decay", "scan_outer", "rotary_pairs_", "gated_group_norm", "qk_unitnorm_store", "window_attn"]
+    saved = {n: getattr(ops, n) for n in names}
+    saved_call = ops.AnyLinear.__call__
+
+    def timed(name, fn):
+        @functools.wraps(fn)
+        def w(*a, **k):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            r = fn(*a, **k)
+            e1.record()
+            times.setdefault(name, []).append((e0, e1))
+            return r
+        return w
+    for n in names:
+        setattr(ops, n, timed(n, saved[n]))
+    ops.AnyLinear.__call__ = timed("linear", saved_call)
+    try:
+        for label, run in (("prefill", lambda: eng.run_ragged([("k", ids, [len(ids) - 1])])),
+                           ("decode", lambda: eng.run_ragged([("k", [5], [0])]))):
+            times.clear()
+            run()
+            torch.cuda.synchronize()
+            tot = {n: sum(a.elapsed_time(b) for a, b in v) for n, v in times.items()}
+            log(f"[bench] width {width} {label}: " + ", ".join(f"{n} {t*1e3:.0f}us x{len(times[n])}" for n, t in
+                                                                sorted(tot.items(), key=lambda kv: -kv[1])))
+        eng.release("k")
+    finally:
+        for n in names:
+            setattr(ops, n, saved[n])
+        ops.AnyLinear.__call__ = saved_call
+
+
 def launch_ranks(args) -> int:
     """The parent of a several-GPU run started without a launcher: N child processes of this file,
     one per rank, as the reference is started (one process per GPU from RANK / WORLD_SIZE,
@@ -610,6 +758,9 @@ def main():
     from micro_vllm_amd.core.layer.sampler import greedy
 
     pc.setup()
+    if args.pagazen:
+        assert world == 1, "--pagazen runs on one GPU"
+        return pagazen_compare(args, dev)
     peers = world > 1                 # ranks to synchronise with
     if args.as_rank_of:
         assert world == 1, "--as-rank-of runs one process"

@@ -43,6 +43,7 @@ class InferenceStats:
 
 
 class InferenceEngine:
+    family = "llama"            # "ragged" once a model of that family has been loaded (models/registry.py)
     DEFAULT_BLOCK_SIZE = 256
     DEFAULT_MAX_BLOCKS = 81
 
@@ -225,7 +226,12 @@ class InferenceEngine:
         if sampling:
             temps = torch.tensor([max(float(s.temperature), 0.0) for s in sampling], device=self.device)
             topp = torch.tensor([float(s.top_p) for s in sampling], device=self.device)
-            picked = self._sample(logits.to(torch.bfloat16), temps, topp, 50)
+            # the sampler reads bf16 rows whose length is a multiple of 8: pad with -inf
+            V = logits.shape[1]
+            rows = torch.full((logits.shape[0], (V + 7) // 8 * 8), float("-inf"), dtype=torch.bfloat16,
+                              device=logits.device)
+            rows[:, :V] = logits
+            picked = self._sample(rows, temps, topp, 50)
             for seq, tok in zip(sampling, picked):
                 seq._next_token = tok
 

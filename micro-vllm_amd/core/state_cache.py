@@ -97,6 +97,10 @@ class HybridCacheManager:
 
     def reserve(self, rows: Seq[Tuple[object, int]]):
         """Slots and pages for one step: rows = [(seq_id, new tokens)].  All or nothing."""
+        for sid, n in rows:
+            if self._len.get(sid, 0) + n > self.max_seq_pages * self.page_size:
+                raise ValueError(f"sequence {sid} would pass the {self.max_seq_pages * self.page_size} positions "
+                                 "a block-table row describes")
         new_slots = len({sid for sid, _ in rows if sid not in self._slot})
         if new_slots > len(self._free_slots):
             raise PoolExhausted(next(sid for sid, _ in rows if sid not in self._slot), "state slot")
@@ -105,9 +109,6 @@ class HybridCacheManager:
             raise PoolExhausted(next(sid for sid, k in need.items() if k), "page")
         for sid, n in rows:
             self.admit(sid)
-            if self._len[sid] + n > self.max_seq_pages * self.page_size:
-                raise ValueError(f"sequence {sid} would pass the {self.max_seq_pages * self.page_size} positions "
-                                 "a block-table row describes")
             for _ in range(need[sid]):
                 self._pages[sid].append(self._free_pages.popleft())
 

@@ -315,7 +315,7 @@ int mv_conv_silu(const float* in, int64_t ldi, float* state, const float* w, con
     using namespace mv;
     if (tokens < 0 || rows < 0 || channels <= 0 || taps < 1 || taps > kMaxTaps) return MV_ERR_INVALID_ARG;
     if (tokens == 0) return MV_OK;
-    if (!in || !state || !w || !out || ldi < channels || ldo < channels) return MV_ERR_INVALID_ARG;
+    if (!in || (!state && taps > 1) || !w || !out || ldi < channels || ldo < channels) return MV_ERR_INVALID_ARG;
     StepRows r{tok_row, nullptr, row_start, row_len, row_ctx, row_slot};
     hipStream_t s = (hipStream_t)stream;
     const int64_t work = (int64_t)tokens * channels;
