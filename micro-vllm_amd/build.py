@@ -51,9 +51,11 @@ FLAGS = [
     "-fno-gpu-rdc",
     "-Wall",
     "-Wno-unused-function",
-    # no packed fp32 arithmetic (v_pk_*_f32): the scalar forms only
-    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
+
+# no packed fp32 arithmetic (v_pk_*_f32), the scalar forms only: for the sources that were written with
+# it.  The older sources keep the flags their kernels were tuned and tested with.
+_NO_PACKED_F32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
 # per-source additions.  attn_prefill.hip: the pipelined attention deals its vector work out slot
@@ -61,6 +63,9 @@ FLAGS = [
 # into one chain of packed additions (slower beside MFMAs than the scalar form, and serial)
 FILE_FLAGS = {
     "attn_prefill.hip": ["-fno-slp-vectorize"],
+    "linear_any.hip": _NO_PACKED_F32,
+    "stream_ops.hip": _NO_PACKED_F32,
+    "seq_mix.hip": _NO_PACKED_F32,
 }
 
 

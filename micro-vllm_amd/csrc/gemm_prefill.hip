@@ -147,13 +147,8 @@ __device__ __forceinline__ void store_wave_tile(const PGemmArgs& a, const f32x4_
         f32x4_t c = acc[i][t];
         for (int e = 0; e < nlower; ++e) {
             f32x4_t part;
-            // the base is the same for every lane; the scalar-register operand needs the compiler to know it
-            const unsigned long long base = (unsigned long long)(lower + (size_t)e * 8 * kWSlotBytes + (i * 8 + t) * 1024);
-            const unsigned long long ubase =
-                ((unsigned long long)__builtin_amdgcn_readfirstlane((unsigned)(base >> 32)) << 32) |
-                (unsigned)__builtin_amdgcn_readfirstlane((unsigned)base);
             asm volatile("global_load_dwordx4 %0, %1, %2 sc1\n\ts_waitcnt vmcnt(0)"
-                         : "=v"(part) : "v"(lane16), "s"((const unsigned char*)ubase) : "memory");
+                         : "=v"(part) : "v"(lane16), "s"(lower + (size_t)e * 8 * kWSlotBytes + (i * 8 + t) * 1024) : "memory");
             c += part;
         }
         return c;
@@ -773,14 +768,11 @@ __device__ __forceinline__ void wide_tile(const PGemmArgs& a, unsigned char* lds
             int nlower = 0;
             if (cur.parts > 1) {
                 if (threadIdx.x == 0) {
-                    // bounded (about 20 s of 0.6-us naps): parts that never arrive mean a lost workgroup,
-                    // and a trap that ends the process beats sums that silently lack a part of k
                     unsigned* const count = &a.cut_count[xcd * wgs + cur.rest];
-                    int spin = 0;
-                    while (__hip_atomic_load(count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (unsigned)(cur.parts - 1)) {
-                        if (++spin > (1 << 25)) __builtin_trap();
+                    for (int spin = 0; spin < (1 << 22) &&
+                                       __hip_atomic_load(count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (unsigned)(cur.parts - 1);
+                         ++spin)
                         __builtin_amdgcn_s_sleep(16);
-                    }
                     __hip_atomic_store(count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
                 __syncthreads();
