@@ -498,19 +498,36 @@ int mv_conv_silu(const float* in, int64_t ldi, float* state, const float* w, con
                  const int32_t* row_ctx, const int32_t* row_slot, int tokens, int rows, int channels, int taps,
                  mv_stream_t stream);
 
-/* gain[t,h] = log(1 + exp(raw[t,h] + dt_bias[h])); decay[t,h] = exp(-exp(a_log[h]) * gain[t,h]). */
+/* gain[t,h] = log(1 + exp(raw[t,h] + dt_bias[h])); log_decay[t,h] = -exp(a_log[h]) * gain[t,h] (may be NULL);
+ * decay[t,h] = exp(log_decay[t,h]). */
 int mv_softplus_decay(const float* raw, int64_t ld, const float* dt_bias, const float* a_log, float* gain,
-                      float* decay, int tokens, int heads, mv_stream_t stream);
+                      float* decay, float* log_decay, int tokens, int heads, mv_stream_t stream);
 
 /* Per row and head, token by token: S = decay[t,h] * S + gain[t,h] * k_t v_t^T (S: n x p, fp32, in
  * state[slot][head]); out[t, h*p ..] = S^T q_t (+ skip[h] * v_t).  q and k of head h are read at
  * column (h / q_div) * n and (h / k_div) * n (heads that share a group); gain == NULL: 1;
- * ld_decay == 0: decay[h] for every token. */
+ * ld_decay == 0: decay[h] for every token.  max_len > 0: rows longer than that are left alone. */
 int mv_scan_outer(const float* q, int64_t ldq, int q_div, const float* k, int64_t ldk, int k_div, const float* v,
                   int64_t ldv, const float* decay, int64_t ld_decay, const float* gain, int64_t ld_gain,
                   const float* skip, float* state, float* out, int64_t ldo, const int32_t* row_start,
                   const int32_t* row_len, const int32_t* row_ctx, const int32_t* row_slot, int rows, int heads, int n,
-                  int p, mv_stream_t stream);
+                  int p, int max_len, mv_stream_t stream);
+
+/* The same recurrence for long rows, 64 tokens at a time (three launches: sums within each chunk, the
+ * states the chunks start from, their contribution to the outputs).  Chunk c covers tokens ch_start[c] ..
+ * + ch_len[c] (<= 64) of one row; row b owns chunks row_ch0[b] .. + row_nch[b] (0: the row is not taken -
+ * mv_scan_outer with max_len > 0 leaves exactly the rows longer than max_len to this call).  The decay
+ * comes as its logarithm ([tokens, heads], or [heads] with ld_ld == 0).  Scratch: ds [chunks, heads, n, p],
+ * lsum [tokens, heads], atot [chunks, heads], all fp32.  Differs from the token-by-token form by the
+ * order of the fp32 sums only.  MV_ERR_UNSUPPORTED when n and p need more LDS than a workgroup has
+ * (mv_scan_chunked_lds_bytes(n, p) > 150 KiB). */
+size_t mv_scan_chunked_lds_bytes(int n, int p);
+int mv_scan_chunked(const float* q, int64_t ldq, int q_div, const float* k, int64_t ldk, int k_div, const float* v,
+                    int64_t ldv, const float* log_decay, int64_t ld_ld, const float* gain, int64_t ld_gain,
+                    const float* skip, float* state, float* out, int64_t ldo, float* ds, float* lsum, float* atot,
+                    const int32_t* ch_start, const int32_t* ch_len, const int32_t* row_ch0, const int32_t* row_nch,
+                    const int32_t* row_ctx, const int32_t* row_slot, int chunks, int rows, int heads, int n, int p,
+                    mv_stream_t stream);
 
 /* In place, per token and head of width dim: (u, v) = (x[i], x[i + rot/2]), i < rot/2, becomes
  * (u cos a - v sin a, v cos a + u sin a), a = tok_pos[t] * inv_freq[i] (formed in fp64); all dim values

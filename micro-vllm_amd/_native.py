@@ -98,9 +98,12 @@ PROTOTYPES = {
     "mv_relu_squared": (_I, [_P, _L, _P, _L, _I, _I, _I, _P]),
     "mv_softcap": (_I, [_P, _L, _F, _P]),
     "mv_conv_silu": (_I, [_P, _L, _P, _P, _P, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
-    "mv_softplus_decay": (_I, [_P, _L, _P, _P, _P, _P, _I, _I, _P]),
+    "mv_softplus_decay": (_I, [_P, _L, _P, _P, _P, _P, _P, _I, _I, _P]),
     "mv_scan_outer": (_I, [_P, _L, _I, _P, _L, _I, _P, _L, _P, _L, _P, _L, _P, _P, _P, _L, _P, _P, _P, _P,
-                           _I, _I, _I, _I, _P]),
+                           _I, _I, _I, _I, _I, _P]),
+    "mv_scan_chunked_lds_bytes": (_Z, [_I, _I]),
+    "mv_scan_chunked": (_I, [_P, _L, _I, _P, _L, _I, _P, _L, _P, _L, _P, _L, _P, _P, _P, _L, _P, _P, _P,
+                             _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "mv_rotary_pairs": (_I, [_P, _L, _P, _P, _I, _I, _I, _I, _F, _P]),
     "mv_gated_group_norm": (_I, [_P, _L, _P, _L, _P, _P, _L, _I, _I, _I, _I, _F, _I, _P]),
     "mv_qk_unitnorm_store": (_I, [_P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P]),

@@ -33,8 +33,12 @@ logger = logging.getLogger(__name__)
 class RaggedRunner:
     PAGE = 64
 
-    def __init__(self, model, device="cuda", dtype=torch.bfloat16, wave_tiles: bool = True):
+    def __init__(self, model, device="cuda", dtype=torch.bfloat16, wave_tiles: bool = True,
+                 chunked_scan: bool = True):
+        """`wave_tiles` / `chunked_scan` = False keep every projection on the plain any-shape kernel and
+        every recurrence token by token (the forms the faster ones are checked against)."""
         assert dtype in (torch.bfloat16, torch.float32)
+        self.chunked_scan = chunked_scan
         self.model, self.cfg, self.device, self.dtype = model, model.config, device, dtype
         self.wave_tiles = wave_tiles
         cfg: PagazenConfig = self.cfg
@@ -81,6 +85,7 @@ class RaggedRunner:
                                              g(p + "mix.right.g")),
                      right_o=self._linear(g(p + "mix.right.o")),
                      decay=self._small(torch.tensor([float(x) for x in R["decay"]], dtype=torch.float64)),
+                     log_decay=self._small(torch.log(torch.tensor([float(x) for x in R["decay"]], dtype=torch.float64))),
                      inv_freq=inv_freq.to(self.device))
             assert len(R["decay"]) == int(R["heads"]), "one decay per retention head"
         if layer.get("mlp"):
@@ -123,12 +128,12 @@ class RaggedRunner:
         proj = w["w_in"](h)                                   # [z | x B C | dt]
         xbc = self._f32buf(T, ch)
         ops.conv_silu(proj[:, inner:inner + ch], st["conv"], w["conv"], w["conv_b"], xbc, step)
-        gain, decay = self._f32buf(T, H), self._f32buf(T, H)
-        ops.softplus_decay(proj[:, inner + ch:inner + ch + H], w["dt_bias"], w["a_log"], gain, decay)
+        gain, decay, log_decay = self._f32buf(T, H), self._f32buf(T, H), self._f32buf(T, H)
+        ops.softplus_decay(proj[:, inner + ch:inner + ch + H], w["dt_bias"], w["a_log"], gain, decay, log_decay)
         y = self._f32buf(T, inner)
         ops.scan_outer(q=xbc[:, inner + G * N:], k=xbc[:, inner:inner + G * N], v=xbc[:, :inner], decay=decay,
                        gain=gain, skip=w["skip"], state=st["ssm"], out=y, step=step, heads=H, n=N, p=P,
-                       q_div=H // G, k_div=H // G)
+                       q_div=H // G, k_div=H // G, log_decay=log_decay, chunked=self.chunked_scan)
         u = self._actbuf(T, inner)
         ops.gated_group_norm(y, proj[:, :inner], w["norm"], u, groups=s["norm_groups"], gate_first=True, eps=eps)
         return w["w_o"](u), None
@@ -152,7 +157,7 @@ class RaggedRunner:
         ops.rotary_pairs_(k, w["inv_freq"], step.tok_pos, Hr, dr, rot, dr ** -0.5)
         o = self._f32buf(T, Hr * dvr)
         ops.scan_outer(q=q, k=k, v=v, decay=w["decay"], gain=None, skip=None, state=cache.states[li]["ret"], out=o,
-                       step=step, heads=Hr, n=dr, p=dvr)
+                       step=step, heads=Hr, n=dr, p=dvr, log_decay=w["log_decay"], chunked=self.chunked_scan)
         u = self._actbuf(T, Hr * dvr)
         ops.gated_group_norm(o, g, None, u, groups=Hr, gate_first=False, eps=eps)
         return left, w["right_o"](u)

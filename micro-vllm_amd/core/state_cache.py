@@ -33,6 +33,16 @@ class RaggedStep:
     block_table: torch.Tensor  # int32 [B, W]
     max_slot: int              # host copies of what the kernels will index with, for the wrappers' checks
     max_page: int
+    # rows of more than SCAN_SEQ_MAX tokens cut into chunks of SCAN_CHUNK for the chunked recurrence
+    n_chunks: int = 0
+    ch_start: torch.Tensor = None   # int32 [chunks] first token of the chunk (index into the step)
+    ch_len: torch.Tensor = None     # int32 [chunks]
+    row_ch0: torch.Tensor = None    # int32 [B] the row's first chunk
+    row_nch: torch.Tensor = None    # int32 [B] its number of chunks (0: a short row)
+
+
+SCAN_CHUNK = 64      # csrc/seq_mix.hip kCh
+SCAN_SEQ_MAX = 16    # rows up to this length run the recurrence token by token
 
 
 class PoolExhausted(RuntimeError):
@@ -67,7 +77,8 @@ class HybridCacheManager:
         self.max_seq_pages = (max_tokens + page_size - 1) // page_size
         self.max_rows, self.max_step_tokens = max_rows, max_step_tokens
         self._on_gpu = torch.cuda.is_available() and str(device).startswith("cuda")
-        words = 3 * max_step_tokens + max_rows * (4 + self.max_seq_pages)
+        words = 3 * max_step_tokens + max_rows * (6 + self.max_seq_pages) + \
+            2 * (max_step_tokens // SCAN_CHUNK + max_rows)
         self._ring = 4 if self._on_gpu else 1
         self._host = [torch.zeros(words, dtype=torch.int32, pin_memory=self._on_gpu) for _ in range(self._ring)]
         self._dev = [torch.zeros(words, dtype=torch.int32, device=device) for _ in range(self._ring)]
@@ -170,7 +181,25 @@ class HybridCacheManager:
             host[o_bt + b * W:o_bt + b * W + len(pages)] = pages
             max_slot, max_page = max(max_slot, slot), max(max_page, max(pages))
             start += n
-        used = o_bt + B * W
+        # chunk table of the long rows
+        o_c0 = o_bt + B * W
+        o_nch = o_c0 + B
+        chunks = []
+        for b, (sid, toks) in enumerate(rows):
+            n = len(toks)
+            host[o_c0 + b] = len(chunks)
+            if n > SCAN_SEQ_MAX:
+                first = int(host[o_rows + b])
+                for off in range(0, n, SCAN_CHUNK):
+                    chunks.append((first + off, min(SCAN_CHUNK, n - off)))
+            host[o_nch + b] = len(chunks) - int(host[o_c0 + b])
+        NC = len(chunks)
+        o_cs = o_nch + B
+        o_cl = o_cs + NC
+        if NC:
+            host[o_cs:o_cs + NC] = [c[0] for c in chunks]
+            host[o_cl:o_cl + NC] = [c[1] for c in chunks]
+        used = o_cl + NC
         dev = self._dev[i]
         dev[:used].copy_(self._host[i][:used], non_blocking=True)
         if self._on_gpu:
@@ -181,4 +210,6 @@ class HybridCacheManager:
             tokens=T, rows=B, page=self.page_size, ids=dev[o_ids:o_ids + T], tok_row=dev[o_row:o_row + T],
             tok_pos=dev[o_pos:o_pos + T], row_start=dev[o_rows:o_rows + B], row_len=dev[o_rows + B:o_rows + 2 * B],
             row_ctx=dev[o_rows + 2 * B:o_rows + 3 * B], row_slot=dev[o_rows + 3 * B:o_rows + 4 * B],
-            block_table=dev[o_bt:o_bt + B * W].view(B, W), max_slot=max_slot, max_page=max_page)
+            block_table=dev[o_bt:o_bt + B * W].view(B, W), max_slot=max_slot, max_page=max_page, n_chunks=NC,
+            ch_start=dev[o_cs:o_cs + NC], ch_len=dev[o_cl:o_cl + NC], row_ch0=dev[o_c0:o_c0 + B],
+            row_nch=dev[o_nch:o_nch + B])

@@ -82,15 +82,17 @@ __global__ __launch_bounds__(256) void conv_state_update_kernel(const float* in,
 }
 
 __global__ __launch_bounds__(256) void softplus_decay_kernel(const float* raw, int64_t ld, const float* dt_bias,
-                                                             const float* a_log, float* gain, float* decay, int T,
-                                                             int H) {
+                                                             const float* a_log, float* gain, float* decay,
+                                                             float* log_decay, int T, int H) {
     const int i = blockIdx.x * 256 + threadIdx.x;
     if (i >= T * H) return;
     const int t = i / H, h = i % H;
     const float v = raw[(int64_t)t * ld + h] + dt_bias[h];
     const float dt = fmaxf(v, 0.f) + log1pf(expf(-fabsf(v)));  // log(1 + e^v), no clamp
     gain[i] = dt;
-    decay[i] = expf(-expf(a_log[h]) * dt);
+    const float ld_ = -expf(a_log[h]) * dt;
+    decay[i] = expf(ld_);
+    if (log_decay) log_decay[i] = ld_;
 }
 
 struct ScanArgs {
@@ -101,6 +103,7 @@ struct ScanArgs {
     float* out;
     StepRows r;
     int H, n, p, pt;
+    int max_len;   // rows longer than this belong to the chunked form (0: every row is taken)
 };
 
 template <int MAXN>
@@ -112,6 +115,7 @@ __global__ __launch_bounds__(256) void scan_outer_kernel(ScanArgs a) {
     const bool vc = c < a.p;
     const int npt = (a.n + NS - 1) / NS, n0 = ng * npt;
     const int len = a.r.row_len[b], start = a.r.row_start[b];
+    if (a.max_len > 0 && len > a.max_len) return;   // the whole workgroup
     const bool carried = a.r.row_ctx[b] > 0;
     float* sp = a.state + (((int64_t)a.r.row_slot[b] * a.H + h) * a.n + n0) * a.p + c;
     float S[MAXN];
@@ -146,6 +150,234 @@ __global__ __launch_bounds__(256) void scan_outer_kernel(ScanArgs a) {
 #pragma unroll
         for (int i = 0; i < MAXN; ++i)
             if (i < npt && n0 + i < a.n) sp[(int64_t)i * a.p] = S[i];
+    }
+}
+
+// ---- the same recurrence in chunks of 64 tokens, for rows long enough to pay for three launches ----
+// Within a chunk that starts from state S0, with L_t the running sum of log decay over the chunk:
+//   o_t = exp(L_t) S0^T q_t + sum_{s<=t} exp(L_t - L_s) gain_s (q_t . k_s) v_s
+//   S_end = exp(L_end) S0 + sum_s exp(L_end - L_s) gain_s k_s v_s^T
+// intra:  per (chunk, head)  the second term of o, the sum of S_end (dS) and exp(L_end), L_t kept
+// carry:  per (row, head)    S0 of every chunk in turn (left where dS was), the row's final state
+// inter:  per (chunk, head)  o_t += exp(L_t) S0^T q_t (+ skip_h v_t)
+// fp32 throughout; differs from the token-by-token form by the order of the sums only.
+constexpr int kCh = 64;
+
+struct ChunkArgs {
+    const float *q, *k, *v, *log_decay, *gain, *skip;
+    int64_t ldq, ldk, ldv, ld_ld, ld_gain, ldo;
+    int q_div, k_div;
+    float* state;
+    float* out;
+    float* ds;     // [chunks, H, n, p]
+    float* lsum;   // [tokens, H]  L_t
+    float* atot;   // [chunks, H]  exp(L_end)
+    const int *ch_start, *ch_len, *row_ch0, *row_nch;
+    StepRows r;
+    int H, n, p;
+};
+
+__global__ __launch_bounds__(256) void scan_chunk_intra_kernel(ChunkArgs a) {
+    extern __shared__ float lds[];
+    const int ch = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int n = a.n, p = a.p, sn = n + 1, sp = p + 1, sc = kCh + 1;
+    float* qs = lds;
+    float* ks = qs + kCh * sn;
+    float* vs = ks + kCh * sn;
+    float* ps = vs + kCh * sp;
+    float* Ls = ps + kCh * sc;
+    float* gs = Ls + kCh;
+    const int start = a.ch_start[ch], len = a.ch_len[ch];
+    for (int i = tid; i < kCh * n; i += 256) {
+        const int t = i / n, j = i % n;
+        const bool ok = t < len;
+        qs[t * sn + j] = ok ? a.q[(int64_t)(start + t) * a.ldq + (int64_t)(h / a.q_div) * n + j] : 0.f;
+        ks[t * sn + j] = ok ? a.k[(int64_t)(start + t) * a.ldk + (int64_t)(h / a.k_div) * n + j] : 0.f;
+    }
+    for (int i = tid; i < kCh * p; i += 256) {
+        const int t = i / p, c = i % p;
+        vs[t * sp + c] = t < len ? a.v[(int64_t)(start + t) * a.ldv + (int64_t)h * p + c] : 0.f;
+    }
+    if (tid < kCh) {   // one wave: inclusive running sum of the log decays
+        float l = 0.f, g = 0.f;
+        if (tid < len) {
+            l = fmaxf(a.log_decay[(int64_t)(start + tid) * a.ld_ld + h], -80.f);
+            g = a.gain ? a.gain[(int64_t)(start + tid) * a.ld_gain + h] : 1.f;
+        }
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const float up = __shfl_up(l, o, 64);
+            if (tid >= o) l += up;
+        }
+        Ls[tid] = l;
+        gs[tid] = g;
+        if (tid < len) a.lsum[(int64_t)(start + tid) * a.H + h] = l;
+    }
+    __syncthreads();
+    const float Lend = Ls[len - 1];
+    if (tid == 0) a.atot[(int64_t)ch * a.H + h] = expf(Lend);
+    const int tt = tid >> 4, cc = tid & 15;
+    // P[t][s] = (q_t . k_s) exp(L_t - L_s) gain_s for s <= t: 4 x 4 entries per thread
+    {
+        const int t0 = tt * 4, s0 = cc * 4;
+        float acc[4][4] = {};
+        if (s0 <= t0 + 3) {
+            for (int j = 0; j < n; ++j) {
+                float qv[4], kv[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    qv[i] = qs[(t0 + i) * sn + j];
+                    kv[i] = ks[(s0 + i) * sn + j];
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[i][e] = fmaf(qv[i], kv[e], acc[i][e]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int t = t0 + i, s_ = s0 + e;
+                ps[t * sc + s_] = (s_ <= t) ? acc[i][e] * expf(Ls[t] - Ls[s_]) * gs[s_] : 0.f;
+            }
+    }
+    __syncthreads();
+    // o[t][c] = sum_s P[t][s] v[s][c]: rows 4 tt .. + 3, columns cc + 16 i
+    for (int c0 = 0; c0 < p; c0 += 128) {
+        float acc[4][8] = {};
+        for (int s_ = 0; s_ < kCh; ++s_) {
+            float pv[4], vv[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) pv[i] = ps[(tt * 4 + i) * sc + s_];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int c = c0 + cc + 16 * e;
+                vv[e] = c < p ? vs[s_ * sp + c] : 0.f;
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[i][e] = fmaf(pv[i], vv[e], acc[i][e]);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int t = tt * 4 + i;
+            if (t >= len) continue;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int c = c0 + cc + 16 * e;
+                if (c < p) a.out[(int64_t)(start + t) * a.ldo + (int64_t)h * p + c] = acc[i][e];
+            }
+        }
+    }
+    // k_s <- k_s exp(L_end - L_s) gain_s, then dS[j][c] = sum_s k[s][j] v[s][c]
+    __syncthreads();
+    for (int i = tid; i < kCh * n; i += 256) {
+        const int t = i / n, j = i % n;
+        ks[t * sn + j] *= expf(Lend - Ls[t]) * gs[t];
+    }
+    __syncthreads();
+    float* dsp = a.ds + ((int64_t)ch * a.H + h) * n * p;
+    for (int j0 = 0; j0 < n; j0 += 64) {
+        for (int c0 = 0; c0 < p; c0 += 128) {
+            float acc[4][8] = {};
+            for (int s_ = 0; s_ < len; ++s_) {
+                float kv[4], vv[8];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int j = j0 + tt + 16 * i;
+                    kv[i] = j < n ? ks[s_ * sn + j] : 0.f;
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int c = c0 + cc + 16 * e;
+                    vv[e] = c < p ? vs[s_ * sp + c] : 0.f;
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) acc[i][e] = fmaf(kv[i], vv[e], acc[i][e]);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int j = j0 + tt + 16 * i;
+                if (j >= n) continue;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int c = c0 + cc + 16 * e;
+                    if (c < p) dsp[(int64_t)j * p + c] = acc[i][e];
+                }
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void scan_chunk_carry_kernel(ChunkArgs a) {
+    const int b = blockIdx.z, h = blockIdx.y;
+    const int np = a.n * a.p, e = blockIdx.x * 256 + threadIdx.x;
+    const int nch = a.row_nch[b];
+    if (nch == 0 || e >= np) return;
+    float* sp = a.state + ((int64_t)a.r.row_slot[b] * a.H + h) * np + e;
+    float S = a.r.row_ctx[b] > 0 ? *sp : 0.f;
+    const int c0 = a.row_ch0[b];
+    for (int c = c0; c < c0 + nch; ++c) {
+        float* d = a.ds + ((int64_t)c * a.H + h) * np + e;
+        const float add = *d;
+        *d = S;                                   // the state this chunk starts from
+        S = fmaf(a.atot[(int64_t)c * a.H + h], S, add);
+    }
+    *sp = S;
+}
+
+__global__ __launch_bounds__(256) void scan_chunk_inter_kernel(ChunkArgs a) {
+    extern __shared__ float lds[];
+    const int ch = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int n = a.n, p = a.p, sn = n + 1, sp = p + 1;
+    float* qs = lds;
+    float* Ss = qs + kCh * sn;
+    const int start = a.ch_start[ch], len = a.ch_len[ch];
+    for (int i = tid; i < kCh * n; i += 256) {
+        const int t = i / n, j = i % n;
+        qs[t * sn + j] = t < len ? a.q[(int64_t)(start + t) * a.ldq + (int64_t)(h / a.q_div) * n + j] : 0.f;
+    }
+    const float* dsp = a.ds + ((int64_t)ch * a.H + h) * n * p;
+    for (int i = tid; i < n * p; i += 256) Ss[(i / p) * sp + i % p] = dsp[i];
+    __syncthreads();
+    const int tt = tid >> 4, cc = tid & 15;
+    const float sk = a.skip ? a.skip[h] : 0.f;
+    for (int c0 = 0; c0 < p; c0 += 128) {
+        float acc[4][8] = {};
+        for (int j = 0; j < n; ++j) {
+            float qv[4], sv[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) qv[i] = qs[(tt * 4 + i) * sn + j];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int c = c0 + cc + 16 * e;
+                sv[e] = c < p ? Ss[j * sp + c] : 0.f;
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[i][e] = fmaf(qv[i], sv[e], acc[i][e]);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int t = tt * 4 + i;
+            if (t >= len) continue;
+            const float w = expf(a.lsum[(int64_t)(start + t) * a.H + h]);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int c = c0 + cc + 16 * e;
+                if (c >= p) continue;
+                float* o = a.out + (int64_t)(start + t) * a.ldo + (int64_t)h * p + c;
+                float r = fmaf(w, acc[i][e], *o);
+                if (a.skip) r = fmaf(sk, a.v[(int64_t)(start + t) * a.ldv + (int64_t)h * p + c], r);
+                *o = r;
+            }
+        }
     }
 }
 
@@ -239,6 +471,10 @@ __global__ __launch_bounds__(256) void qk_unitnorm_store_kernel(float* qkv, int6
 
 constexpr int kMaxVC = 4;  // value columns per lane: vdim <= 256
 
+// One workgroup per (token, head).  Its four waves take the window's 64-key tiles in turn: a lane scores
+// one key (q from LDS, the key row straight from its page), the wave forms max / sum of the tile and
+// then, lanes now owning value columns, adds the tile's weighted values; the waves' partial softmaxes
+// meet in LDS.  The same code serves a prompt's portion and a single decoded token.
 template <bool F32>
 __global__ __launch_bounds__(256) void window_attn_kernel(const float* q, int64_t ldq, const void* kc_,
                                                           const void* vc_, void* out_, int64_t ldo, PagedRows pr,
@@ -250,35 +486,48 @@ __global__ __launch_bounds__(256) void window_attn_kernel(const float* q, int64_
     const T_* vc = (const T_*)vc_;
     T_* out = (T_*)out_;
     const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    float* qs = lds + wv * (d + 64);
-    float* ps = qs + d;
-    const int64_t unit = (int64_t)blockIdx.x * 4 + wv;
-    if (unit >= (int64_t)T * H) return;   // whole waves leave; no block-wide barrier below
-    const int t = (int)(unit / H), h = (int)(unit % H), g = h / (H / G);
+    float* qs = lds;
+    float* ps = lds + d + wv * 64;
+    float* mm = lds + d + 256;
+    float* ll = mm + 4;
+    float* aa = ll + 4;
+    const int t = blockIdx.x / H, h = blockIdx.x % H, g = h / (H / G);
     const int pos = pr.tok_pos[t];
     const int* bt = pr.block_table + (int64_t)pr.tok_row[t] * pr.bt_stride;
     const int lo = pos - window + 1 > 0 ? pos - window + 1 : 0;
     const float slope = slopes ? slopes[h] : 0.f;
-    for (int c = lane; c < d; c += 64) qs[c] = q[(int64_t)t * ldq + (int64_t)h * d + c];
-    __builtin_amdgcn_wave_barrier();   // qs and ps are exchanged between the lanes of this wave only
+    for (int c = threadIdx.x; c < d; c += 256) qs[c] = q[(int64_t)t * ldq + (int64_t)h * d + c];
+    __syncthreads();
     float m = -INFINITY, l = 0.f, acc[kMaxVC] = {0.f, 0.f, 0.f, 0.f};
-    for (int j0 = lo; j0 <= pos; j0 += 64) {
+    for (int j0 = lo + 64 * wv; j0 <= pos; j0 += 256) {
         const int j = j0 + lane;
         float s = -INFINITY;
         if (j <= pos) {
             const int pg = bt[j / pr.page];
             const T_* kr = kc + (((int64_t)pg * pr.page + j % pr.page) * G + g) * d;
             float dot = 0.f;
-            for (int c = 0; c < d; ++c) dot = fmaf(qs[c], ActS<F32>::ld(kr + c), dot);
+            if (!F32 && (d & 7) == 0) {
+                for (int c = 0; c < d; c += 8) {
+                    const uint4 kv = ld16(kr + c);
+                    const uint32_t w[4] = {kv.x, kv.y, kv.z, kv.w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        dot = fmaf(qs[c + 2 * e], bf16_lo(w[e]), dot);
+                        dot = fmaf(qs[c + 2 * e + 1], bf16_hi(w[e]), dot);
+                    }
+                }
+            } else {
+                for (int c = 0; c < d; ++c) dot = fmaf(qs[c], ActS<F32>::ld(kr + c), dot);
+            }
             s = dot * scale - slope * (float)(pos - j);
         }
         const float mn = fmaxf(m, wave_max(s));
-        const float p = j <= pos ? expf(s - mn) : 0.f;
-        const float corr = expf(m - mn);   // m = -inf on the first tile: exp(-inf) = 0
-        l = l * corr + wave_sum(p);
+        const float pj_ = j <= pos ? expf(s - mn) : 0.f;
+        const float corr = expf(m - mn);   // m = -inf on the wave's first tile: exp(-inf) = 0
+        l = l * corr + wave_sum(pj_);
         m = mn;
         __builtin_amdgcn_wave_barrier();
-        ps[lane] = p;
+        ps[lane] = pj_;
         __builtin_amdgcn_wave_barrier();
         const int cnt = pos - j0 + 1 < 64 ? pos - j0 + 1 : 64;
 #pragma unroll
@@ -295,10 +544,60 @@ __global__ __launch_bounds__(256) void window_attn_kernel(const float* q, int64_
             }
         }
     }
+    if (lane == 0) {
+        mm[wv] = m;
+        ll[wv] = l;
+    }
 #pragma unroll
     for (int ci = 0; ci < kMaxVC; ++ci) {
         const int c = lane + ci * 64;
-        if (c < dv) ActS<F32>::st(out + (int64_t)t * ldo + (int64_t)h * dv + c, acc[ci] / l);
+        if (c < dv) aa[wv * dv + c] = acc[ci];
+    }
+    __syncthreads();
+    if (wv == 0) {
+        float M = fmaxf(fmaxf(mm[0], mm[1]), fmaxf(mm[2], mm[3]));   // wave 0 always has a key: finite
+        float w4[4], L = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            w4[w] = expf(mm[w] - M);   // a wave without keys: exp(-inf) = 0
+            L = fmaf(ll[w], w4[w], L);
+        }
+#pragma unroll
+        for (int ci = 0; ci < kMaxVC; ++ci) {
+            const int c = lane + ci * 64;
+            if (c < dv) {
+                float o = 0.f;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) o = fmaf(aa[w * dv + c], w4[w], o);
+                ActS<F32>::st(out + (int64_t)t * ldo + (int64_t)h * dv + c, o / L);
+            }
+        }
+    }
+}
+
+// groups of a thousand values and more: one workgroup per (row, group)
+template <bool F32>
+__global__ __launch_bounds__(256) void gated_group_norm_wide_kernel(const float* y, int64_t ldy, const float* gate,
+                                                                    int64_t ldg, const float* w, void* out_,
+                                                                    int64_t ldo, int n, int groups, int gate_first,
+                                                                    float eps) {
+    typedef typename ActS<F32>::T T;
+    __shared__ float red[4];
+    T* out = (T*)out_;
+    const int row = blockIdx.x / groups, g = blockIdx.x % groups, gs = n / groups;
+    const float* yr = y + (int64_t)row * ldy + (int64_t)g * gs;
+    const float* gr = gate + (int64_t)row * ldg + (int64_t)g * gs;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < gs; c += 256) {
+        const float u = gate_first ? yr[c] * silu_f(gr[c]) : yr[c];
+        ss += u * u;
+    }
+    ss = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)gs + eps);
+    for (int c = threadIdx.x; c < gs; c += 256) {
+        float u = gate_first ? (yr[c] * silu_f(gr[c])) * inv : (yr[c] * inv) * silu_f(gr[c]);
+        if (w) u *= w[g * gs + c];
+        ActS<F32>::st(out + (int64_t)row * ldo + (int64_t)g * gs + c, u);
     }
 }
 
@@ -330,13 +629,13 @@ int mv_conv_silu(const float* in, int64_t ldi, float* state, const float* w, con
 }
 
 int mv_softplus_decay(const float* raw, int64_t ld, const float* dt_bias, const float* a_log, float* gain,
-                      float* decay, int tokens, int heads, mv_stream_t stream) {
+                      float* decay, float* log_decay, int tokens, int heads, mv_stream_t stream) {
     using namespace mv;
     if (tokens < 0 || heads <= 0) return MV_ERR_INVALID_ARG;
     if (tokens == 0) return MV_OK;
     if (!raw || !dt_bias || !a_log || !gain || !decay || ld < heads) return MV_ERR_INVALID_ARG;
     hipLaunchKernelGGL(softplus_decay_kernel, dim3((tokens * heads + 255) / 256), dim3(256), 0, (hipStream_t)stream,
-                       raw, ld, dt_bias, a_log, gain, decay, tokens, heads);
+                       raw, ld, dt_bias, a_log, gain, decay, log_decay, tokens, heads);
     return check_launch();
 }
 
@@ -344,7 +643,7 @@ int mv_scan_outer(const float* q, int64_t ldq, int q_div, const float* k, int64_
                   int64_t ldv, const float* decay, int64_t ld_decay, const float* gain, int64_t ld_gain,
                   const float* skip, float* state, float* out, int64_t ldo, const int32_t* row_start,
                   const int32_t* row_len, const int32_t* row_ctx, const int32_t* row_slot, int rows, int heads, int n,
-                  int p, mv_stream_t stream) {
+                  int p, int max_len, mv_stream_t stream) {
     using namespace mv;
     if (rows < 0 || heads <= 0 || n <= 0 || p <= 0 || q_div <= 0 || k_div <= 0) return MV_ERR_INVALID_ARG;
     if (rows == 0) return MV_OK;
@@ -354,7 +653,7 @@ int mv_scan_outer(const float* q, int64_t ldq, int q_div, const float* k, int64_
     a.ldq = ldq; a.ldk = ldk; a.ldv = ldv; a.ld_decay = ld_decay; a.ld_gain = ld_gain; a.ldo = ldo;
     a.q_div = q_div; a.k_div = k_div; a.state = state; a.out = out;
     a.r = StepRows{nullptr, nullptr, row_start, row_len, row_ctx, row_slot};
-    a.H = heads; a.n = n; a.p = p;
+    a.H = heads; a.n = n; a.p = p; a.max_len = max_len;
     a.pt = p % 64 == 0 ? 64 : (p % 32 == 0 ? 32 : 16);
     const int ns = 256 / a.pt, npt = (n + ns - 1) / ns;
     const dim3 grid((p + a.pt - 1) / a.pt, heads, rows);
@@ -363,6 +662,42 @@ int mv_scan_outer(const float* q, int64_t ldq, int q_div, const float* k, int64_
     else if (npt <= 16) hipLaunchKernelGGL(scan_outer_kernel<16>, grid, dim3(256), 0, s, a);
     else if (npt <= 64) hipLaunchKernelGGL(scan_outer_kernel<64>, grid, dim3(256), 0, s, a);
     else return MV_ERR_UNSUPPORTED;
+    return check_launch();
+}
+
+size_t mv_scan_chunked_lds_bytes(int n, int p) {
+    return (size_t)(2 * mv::kCh * (n + 1) + mv::kCh * (p + 1) + mv::kCh * (mv::kCh + 1) + 2 * mv::kCh) * sizeof(float);
+}
+
+int mv_scan_chunked(const float* q, int64_t ldq, int q_div, const float* k, int64_t ldk, int k_div, const float* v,
+                    int64_t ldv, const float* log_decay, int64_t ld_ld, const float* gain, int64_t ld_gain,
+                    const float* skip, float* state, float* out, int64_t ldo, float* ds, float* lsum, float* atot,
+                    const int32_t* ch_start, const int32_t* ch_len, const int32_t* row_ch0, const int32_t* row_nch,
+                    const int32_t* row_ctx, const int32_t* row_slot, int chunks, int rows, int heads, int n, int p,
+                    mv_stream_t stream) {
+    using namespace mv;
+    if (chunks < 0 || rows < 0 || heads <= 0 || n <= 0 || p <= 0 || q_div <= 0 || k_div <= 0) return MV_ERR_INVALID_ARG;
+    if (chunks == 0) return MV_OK;
+    if (!q || !k || !v || !log_decay || !state || !out || !ds || !lsum || !atot || !ch_start || !ch_len || !row_ch0 ||
+        !row_nch || rows > 65535 || heads > 65535)
+        return MV_ERR_INVALID_ARG;
+    const size_t lds = mv_scan_chunked_lds_bytes(n, p);
+    const size_t lds2 = (size_t)(kCh * (n + 1) + n * (p + 1)) * sizeof(float);
+    if (lds > 150 * 1024 || lds2 > 150 * 1024) return MV_ERR_UNSUPPORTED;
+    static LdsOptIn opt1, opt2;
+    if (int rc = ensure_dynamic_lds((const void*)scan_chunk_intra_kernel, lds, opt1)) return rc;
+    if (int rc = ensure_dynamic_lds((const void*)scan_chunk_inter_kernel, lds2, opt2)) return rc;
+    ChunkArgs a;
+    a.q = q; a.k = k; a.v = v; a.log_decay = log_decay; a.gain = gain; a.skip = skip;
+    a.ldq = ldq; a.ldk = ldk; a.ldv = ldv; a.ld_ld = ld_ld; a.ld_gain = ld_gain; a.ldo = ldo;
+    a.q_div = q_div; a.k_div = k_div; a.state = state; a.out = out; a.ds = ds; a.lsum = lsum; a.atot = atot;
+    a.ch_start = ch_start; a.ch_len = ch_len; a.row_ch0 = row_ch0; a.row_nch = row_nch;
+    a.r = StepRows{nullptr, nullptr, nullptr, nullptr, row_ctx, row_slot};
+    a.H = heads; a.n = n; a.p = p;
+    hipStream_t s = (hipStream_t)stream;
+    hipLaunchKernelGGL(scan_chunk_intra_kernel, dim3(chunks, heads), dim3(256), lds, s, a);
+    hipLaunchKernelGGL(scan_chunk_carry_kernel, dim3((n * p + 255) / 256, heads, rows), dim3(256), 0, s, a);
+    hipLaunchKernelGGL(scan_chunk_inter_kernel, dim3(chunks, heads), dim3(256), lds2, s, a);
     return check_launch();
 }
 
@@ -386,8 +721,14 @@ int mv_gated_group_norm(const float* y, int64_t ldy, const float* gate, int64_t 
     if (rows == 0) return MV_OK;
     if (!y || !gate || !out || ldy < n || ldg < n || ldo < n) return MV_ERR_INVALID_ARG;
     const int64_t units = (int64_t)rows * groups;
-    const dim3 grid((unsigned)((units + 3) / 4));
     hipStream_t s = (hipStream_t)stream;
+    if (n / groups >= 1024) {
+        const dim3 wide((unsigned)units);
+        if (f32) hipLaunchKernelGGL(gated_group_norm_wide_kernel<true>, wide, dim3(256), 0, s, y, ldy, gate, ldg, w, out, ldo, n, groups, gate_first, eps);
+        else hipLaunchKernelGGL(gated_group_norm_wide_kernel<false>, wide, dim3(256), 0, s, y, ldy, gate, ldg, w, out, ldo, n, groups, gate_first, eps);
+        return check_launch();
+    }
+    const dim3 grid((unsigned)((units + 3) / 4));
     if (f32) hipLaunchKernelGGL(gated_group_norm_kernel<true>, grid, dim3(256), 0, s, y, ldy, gate, ldg, w, out, ldo, rows, n, groups, gate_first, eps);
     else hipLaunchKernelGGL(gated_group_norm_kernel<false>, grid, dim3(256), 0, s, y, ldy, gate, ldg, w, out, ldo, rows, n, groups, gate_first, eps);
     return check_launch();
@@ -425,8 +766,9 @@ int mv_window_attn(const float* q, int64_t ldq, const void* k_cache, const void*
     if (!q || !k_cache || !v_cache || !out || !tok_row || !tok_pos || !block_table) return MV_ERR_INVALID_ARG;
     PagedRows pr{tok_row, tok_pos, block_table, bt_stride, page};
     const int64_t units = (int64_t)tokens * heads;
-    const dim3 grid((unsigned)((units + 3) / 4));
-    const size_t lds = (size_t)4 * (d + 64) * sizeof(float);
+    if (units > 0x7fffffff) return MV_ERR_UNSUPPORTED;
+    const dim3 grid((unsigned)units);
+    const size_t lds = (size_t)(d + 256 + 8 + 4 * dv) * sizeof(float);
     hipStream_t s = (hipStream_t)stream;
     if (f32) hipLaunchKernelGGL(window_attn_kernel<true>, grid, dim3(256), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window);
     else hipLaunchKernelGGL(window_attn_kernel<false>, grid, dim3(256), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window);

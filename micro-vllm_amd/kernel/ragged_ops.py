@@ -129,19 +129,24 @@ def conv_silu(inp, state, w, bias, out, step):
         step.row_slot.data_ptr(), tokens, step.rows, ch, taps, nv.stream_ptr()))
 
 
-def softplus_decay(raw, dt_bias, a_log, gain, decay):
+def softplus_decay(raw, dt_bias, a_log, gain, decay, log_decay=None):
     tokens, heads = raw.shape
     assert gain.shape == (tokens, heads) and decay.shape == (tokens, heads)
     assert gain.is_contiguous() and decay.is_contiguous() and dt_bias.numel() == heads and a_log.numel() == heads
+    assert log_decay is None or (log_decay.shape == (tokens, heads) and log_decay.is_contiguous())
     nv.check("mv_softplus_decay", nv.lib().mv_softplus_decay(
         _f32(raw).data_ptr(), _ld(raw), _f32(dt_bias).data_ptr(), _f32(a_log).data_ptr(), _f32(gain).data_ptr(),
-        _f32(decay).data_ptr(), tokens, heads, nv.stream_ptr()))
+        _f32(decay).data_ptr(), None if log_decay is None else _f32(log_decay).data_ptr(), tokens, heads,
+        nv.stream_ptr()))
 
 
 def scan_outer(q, k, v, decay, gain, skip, state, out, step, heads: int, n: int, p: int, q_div: int = 1,
-               k_div: int = 1):
+               k_div: int = 1, log_decay=None, chunked: bool = True):
     """state [slots, heads, n, p] fp32; q [T, heads/q_div * n], k [T, heads/k_div * n], v and out
-    [T, heads * p]; decay [T, heads] or [heads] (the same for every token); gain [T, heads] or None."""
+    [T, heads * p]; decay [T, heads] or [heads] (the same for every token); gain [T, heads] or None.
+    Rows of up to SCAN_SEQ_MAX tokens run token by token; with `log_decay` (the decay's logarithm, shaped
+    like it) longer rows run in chunks of 64 (mv_scan_chunked) unless `chunked` is False or the head
+    shape does not fit a workgroup's LDS."""
     tokens = v.shape[0]
     assert q.shape == (tokens, heads // q_div * n) and k.shape == (tokens, heads // k_div * n)
     assert v.shape == (tokens, heads * p) and out.shape == (tokens, heads * p)
@@ -155,13 +160,31 @@ def scan_outer(q, k, v, decay, gain, skip, state, out, step, heads: int, n: int,
         ld_decay = _ld(decay)
     assert gain is None or gain.shape == (tokens, heads)
     assert skip is None or (skip.numel() == heads and skip.is_contiguous())
+    L = nv.lib()
+    use_chunks = (chunked and log_decay is not None and step.n_chunks > 0
+                  and L.mv_scan_chunked_lds_bytes(n, p) <= 150 * 1024 and (64 * (n + 1) + n * (p + 1)) * 4 <= 150 * 1024)
+    if use_chunks:
+        assert log_decay.shape == decay.shape and log_decay.stride(-1) == 1
+        dev = v.device
+        ds = torch.empty(step.n_chunks, heads, n, p, dtype=torch.float32, device=dev)
+        lsum = torch.empty(tokens, heads, dtype=torch.float32, device=dev)
+        atot = torch.empty(step.n_chunks, heads, dtype=torch.float32, device=dev)
+        nv.check("mv_scan_chunked", L.mv_scan_chunked(
+            _f32(q).data_ptr(), _ld(q), q_div, _f32(k).data_ptr(), _ld(k), k_div, _f32(v).data_ptr(), _ld(v),
+            _f32(log_decay).data_ptr(), 0 if log_decay.dim() == 1 else _ld(log_decay),
+            None if gain is None else _f32(gain).data_ptr(), 0 if gain is None else _ld(gain),
+            None if skip is None else _f32(skip).data_ptr(), _f32(state).data_ptr(), _f32(out).data_ptr(), _ld(out),
+            ds.data_ptr(), lsum.data_ptr(), atot.data_ptr(), step.ch_start.data_ptr(), step.ch_len.data_ptr(),
+            step.row_ch0.data_ptr(), step.row_nch.data_ptr(), step.row_ctx.data_ptr(), step.row_slot.data_ptr(),
+            step.n_chunks, step.rows, heads, n, p, nv.stream_ptr()))
+    from ..core.state_cache import SCAN_SEQ_MAX
     nv.check("mv_scan_outer", nv.lib().mv_scan_outer(
         _f32(q).data_ptr(), _ld(q), q_div, _f32(k).data_ptr(), _ld(k), k_div, _f32(v).data_ptr(), _ld(v),
         _f32(decay).data_ptr(), ld_decay, None if gain is None else _f32(gain).data_ptr(),
         0 if gain is None else _ld(gain), None if skip is None else _f32(skip).data_ptr(),
         _f32(state).data_ptr(), _f32(out).data_ptr(), _ld(out), step.row_start.data_ptr(),
         step.row_len.data_ptr(), step.row_ctx.data_ptr(), step.row_slot.data_ptr(), step.rows, heads, n, p,
-        nv.stream_ptr()))
+        SCAN_SEQ_MAX if use_chunks else 0, nv.stream_ptr()))
 
 
 def rotary_pairs_(x, inv_freq, tok_pos, heads: int, dim: int, rot: int, scale: float = 1.0):

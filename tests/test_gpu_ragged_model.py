@@ -56,8 +56,22 @@ def test_portions_and_decoding_match_the_whole_prompt_fp32(make):
     assert rel_err(whole, want) < 1e-4
     for portions in ([1] * 140, [2] * 70, [3, 2, 64, 5, 2, 64], [63, 1, 1, 75], [64, 64, 12], [100] + [1] * 40):
         got = run_in_portions(eng, "p", toks, portions)
-        assert rel_err(got, whole) < 2e-6, portions       # the same sums in the same order
+        assert rel_err(got, whole) < 2e-5, portions       # the same sums, in another order where a recurrence is chunked
         assert rel_err(got, want) < 1e-4, portions
+
+
+def test_token_by_token_forms_agree_with_the_fast_ones():
+    """The plain any-shape projection and the token-by-token recurrence against the wave-tile projections
+    and the chunked recurrence the runner takes by default."""
+    from micro_vllm_amd.core.layer.ragged_runner import RaggedRunner
+    cfg = config_b()
+    toks = tokens_for(cfg, 200, 15)
+    for dtype, tol in ((torch.float32, 2e-5), (torch.bfloat16, 2e-2)):
+        eng = make_engine(cfg, dtype)
+        fast = run_in_portions(eng, "f", toks, [130, 70])
+        eng.runner = RaggedRunner(eng.model, eng.device, dtype, wave_tiles=False, chunked_scan=False)
+        slow = run_in_portions(eng, "s", toks, [130, 70])
+        assert rel_err(fast, slow) < tol
 
 
 def test_first_tokens_fp32():
@@ -95,7 +109,7 @@ def test_mixed_batch_equals_each_request_alone_fp32():
                 eng.release(k)
     for k in reqs:
         assert at[k] == len(reqs[k])
-        assert rel_err(torch.cat(got[k]), alone[k]) < 2e-6, k
+        assert rel_err(torch.cat(got[k]), alone[k]) < 2e-5, k
 
 
 def test_pages_and_slots_used_again_fp32():
@@ -111,7 +125,7 @@ def test_pages_and_slots_used_again_fp32():
         eng.run_ragged([("c", c[:5], [])])
     eng.release("a")                                                   # its pages and slot hold a's data
     got = run_in_portions(eng, "c", c, [7, 64, 49], release=False)
-    assert rel_err(got, ref_c) < 2e-6
+    assert rel_err(got, ref_c) < 2e-5
     eng.release("b")
     eng.release("c")
     assert eng.cache_manager.stats["free"] == 6 and eng.cache_manager.stats["slots_free"] == 2

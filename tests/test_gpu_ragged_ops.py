@@ -116,12 +116,14 @@ def test_softplus_decay(ops):
     g = torch.Generator().manual_seed(5)
     raw = torch.randn(9, 11, generator=g) * 30         # far into both tails: no clamp anywhere
     bias, a_log = torch.randn(5, generator=g), torch.randn(5, generator=g)
-    gain, decay = torch.empty(9, 5, device=DEV), torch.empty(9, 5, device=DEV)
-    ops.softplus_decay(raw.to(DEV)[:, 4:9], bias.to(DEV), a_log.to(DEV), gain, decay)
+    gain, decay, logd = torch.empty(9, 5, device=DEV), torch.empty(9, 5, device=DEV), torch.empty(9, 5, device=DEV)
+    ops.softplus_decay(raw.to(DEV)[:, 4:9], bias.to(DEV), a_log.to(DEV), gain, decay, logd)
     v = raw[:, 4:9].double() + bias.double()
     dt = torch.where(v > 30, v, torch.log1p(torch.exp(v)))
     assert ((gain.cpu().double() - dt).abs() / dt.abs().clamp_min(1e-30)).max().item() < 1e-5
     assert (decay.cpu().double() - torch.exp(-torch.exp(a_log.double()) * dt)).abs().max().item() < 1e-6
+    want = -torch.exp(a_log.double()) * dt
+    assert ((logd.cpu().double() - want).abs() / want.abs().clamp_min(1e-30)).max().item() < 1e-5
 
 
 @pytest.mark.parametrize("H,G,n,p", [(4, 2, 40, 24), (3, 3, 48, 20), (2, 1, 128, 64), (1, 1, 8, 128), (6, 1, 48, 48)])
@@ -163,6 +165,51 @@ def test_scan_whole_portions_and_rows(ops, H, G, n, p):
                                                v[lo:hi].double().view(-1, H, p), decay[0].double().repeat(hi - lo, 1),
                                                torch.ones(hi - lo, H, dtype=torch.float64))
         assert (o[lo:hi].cpu().double() - w2.reshape(hi - lo, H * p)).abs().max().item() < 2e-4
+
+
+@pytest.mark.parametrize("H,G,n,p", [(4, 2, 40, 24), (2, 1, 128, 64), (1, 1, 8, 130), (3, 3, 64, 32)])
+def test_scan_in_chunks_equals_token_by_token(ops, H, G, n, p):
+    """Long rows: the chunked form against the restatement and against the token-by-token kernel, whole
+    and cut at places that are no multiple of the chunk, beside a short row in the same launch; decays
+    from nearly one down to values whose products underflow."""
+    g = torch.Generator().manual_seed(H * 7 + p)
+    T, rep = 333, H // G
+    q, k = torch.randn(T, G * n, generator=g), torch.randn(T, G * n, generator=g)
+    v = torch.randn(T, H * p, generator=g)
+    logd = -torch.exp(torch.randn(T, H, generator=g) * 3.0 - 3.0)
+    logd[100:110] = -120.0                       # a stretch that forgets everything
+    decay, gain = torch.exp(logd), torch.rand(T, H, generator=g) + 0.1
+    skip = torch.randn(H, generator=g)
+    want, _ = ref.decayed_outer_product_scan(
+        q.double().view(T, G, n).repeat_interleave(rep, 1), k.double().view(T, G, n).repeat_interleave(rep, 1),
+        v.double().view(T, H, p), torch.exp(logd.double()), gain.double())
+    want = (want + skip.double()[None, :, None] * v.double().view(T, H, p)).reshape(T, H * p)
+    dv = lambda t: t.to(DEV)
+    outs = {}
+    for chunked in (True, False):
+        for portions in ([T], [70, 3, 129, 17, 64, 50], [200] + [1] * 133):
+            cache = make_cache(state={0: {"s": (H, n, p)}})
+            cache.admit("other")
+            cache.states[0]["s"].fill_(3.0)
+            out, pos = [], 0
+            for m in portions:
+                rows = [("a", [0] * m)] + ([("b", [0] * 5)] if pos == 0 else [])     # a short row rides along once
+                st = step_of(cache, rows)
+                if chunked:
+                    assert st.n_chunks == (m + 63) // 64 * (m > 16)
+                tot = st.tokens
+                o = torch.empty(tot, H * p, device=DEV)
+                pad = lambda t: torch.cat([t[pos:pos + m], t[:tot - m]]).to(DEV)
+                ops.scan_outer(pad(q), pad(k), pad(v), pad(decay), pad(gain), dv(skip), cache.states[0]["s"], o, st,
+                               H, n, p, q_div=rep, k_div=rep, log_decay=pad(logd), chunked=chunked)
+                out.append(o[:m].cpu())
+                if pos == 0:
+                    assert (o[m:].cpu().double() - want[:5]).abs().max().item() < 2e-4
+                pos += m
+            got = torch.cat(out).double()
+            assert (got - want).abs().max().item() < 5e-4 * max(1.0, want.abs().max().item()), (chunked, portions)
+            outs[(chunked, len(portions))] = got
+    assert (outs[(True, 1)] - outs[(False, 1)]).abs().max().item() < 5e-4 * max(1.0, want.abs().max().item())
 
 
 @pytest.mark.parametrize("dim,rot", [(48, 32), (64, 64), (40, 0), (6, 2)])

@@ -71,6 +71,9 @@ def test_pages_slots_and_step_layout(mv):
     assert sorted(st.row_slot.tolist()) == [0, 1]
     assert st.block_table[0, :2].tolist() == c.get_blocks("a") and st.block_table[0, 2].item() == -1
     assert c.stats["free"] == 2
+    # the long row is cut into chunks of 64 for the chunked recurrence, the short one is not
+    assert st.n_chunks == 2 and st.ch_start.tolist() == [0, 64] and st.ch_len.tolist() == [64, 6]
+    assert st.row_ch0.tolist() == [0, 2] and st.row_nch.tolist() == [2, 0]
     c.reserve([("a", 58)])                       # fills its second page exactly: no new page
     assert c.stats["free"] == 2
     st = c.plan([("a", [1] * 58)])
