@@ -323,13 +323,20 @@ def main(argv=None):
                     help="share of the free device memory the KV pool takes when --kv-blocks is not given")
     ap.add_argument("--exact-rope", action="store_true")
     ap.add_argument("--trust-remote-code", action="store_true", help="for tokenizers shipped as Python")
+    ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16",
+                    help="float32: the whole model in 32 bits (model families with ragged steps only)")
+    ap.add_argument("--state-slots", type=int, default=None,
+                    help="recurrent-state slots of a model family with ragged steps (default: --max-batch-size)")
     args = ap.parse_args(argv)
 
+    import torch
     from .core.engine import InferenceEngine
     engine = InferenceEngine(args.model_path, args.max_batch_size, args.max_prefill_tokens,
                              n_blocks=args.kv_blocks if args.kv_blocks is not None else "auto",
                              kv_fraction=args.kv_fraction, max_tokens=args.max_tokens,
-                             exact_rope=args.exact_rope, trust_remote_code=args.trust_remote_code)
+                             exact_rope=args.exact_rope, trust_remote_code=args.trust_remote_code,
+                             dtype=torch.float32 if args.dtype == "float32" else torch.bfloat16,
+                             state_slots=args.state_slots)
     loop = EngineLoop(engine)
     logger.info("rank %d: model loaded on %s", get_rank(), engine.device)
     if not rank0():

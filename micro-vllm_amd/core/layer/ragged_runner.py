@@ -34,11 +34,16 @@ class RaggedRunner:
     PAGE = 64
 
     def __init__(self, model, device="cuda", dtype=torch.bfloat16, wave_tiles: bool = True,
-                 chunked_scan: bool = True):
+                 chunked_scan: bool = True, graphs: bool = True, max_graph_rows: int = 64):
         """`wave_tiles` / `chunked_scan` = False keep every projection on the plain any-shape kernel and
-        every recurrence token by token (the forms the faster ones are checked against)."""
+        every recurrence token by token (the forms the faster ones are checked against).  `graphs`:
+        steps in which every row brings one token (decoding) are captured once per row count into a
+        hipGraph and replayed - some seventy launches become one."""
         assert dtype in (torch.bfloat16, torch.float32)
         self.chunked_scan = chunked_scan
+        self.use_graphs, self.max_graph_rows = graphs, max_graph_rows
+        self._graphs: Dict[int, tuple] = {}
+        self._arena, self._arena_off, self._measured = None, 0, 0
         self.model, self.cfg, self.device, self.dtype = model, model.config, device, dtype
         self.wave_tiles = wave_tiles
         cfg: PagazenConfig = self.cfg
@@ -115,17 +120,29 @@ class RaggedRunner:
                                   max_tokens=max_tokens, max_rows=max_rows, max_step_tokens=max_step_tokens)
 
     # ------------------------------------------------------------------ layers
+    def _take(self, rows, cols, dtype):
+        """A [rows, cols] buffer: from the arena of the step being captured or replayed (the same
+        addresses every time), else a fresh allocation."""
+        nbytes = (rows * cols * (4 if dtype == torch.float32 else 2) + 255) // 256 * 256
+        self._measured += nbytes
+        if self._arena is None:
+            return torch.empty(rows, cols, dtype=dtype, device=self.device)
+        assert self._arena_off + nbytes <= self._arena.numel(), "step arena too small"
+        t = self._arena[self._arena_off:self._arena_off + nbytes].view(dtype)[:rows * cols].view(rows, cols)
+        self._arena_off += nbytes
+        return t
+
     def _f32buf(self, rows, cols):
-        return torch.empty(rows, cols, dtype=torch.float32, device=self.device)
+        return self._take(rows, cols, torch.float32)
 
     def _actbuf(self, rows, cols):
-        return torch.empty(rows, cols, dtype=self.dtype, device=self.device)
+        return self._take(rows, cols, self.dtype)
 
     def _mamba2(self, li, w, h, step: RaggedStep, cache: HybridCacheManager):
         s, T, eps = w["sizes"], step.tokens, self.cfg.eps
         inner, ch, H, N, P, G = s["inner"], s["conv_ch"], s["heads"], s["n"], s["p"], s["groups"]
         st = cache.states[li]
-        proj = w["w_in"](h)                                   # [z | x B C | dt]
+        proj = w["w_in"](h, self._f32buf(T, w["w_in"].n))     # [z | x B C | dt]
         xbc = self._f32buf(T, ch)
         ops.conv_silu(proj[:, inner:inner + ch], st["conv"], w["conv"], w["conv_b"], xbc, step)
         gain, decay, log_decay = self._f32buf(T, H), self._f32buf(T, H), self._f32buf(T, H)
@@ -136,21 +153,21 @@ class RaggedRunner:
                        q_div=H // G, k_div=H // G, log_decay=log_decay, chunked=self.chunked_scan)
         u = self._actbuf(T, inner)
         ops.gated_group_norm(y, proj[:, :inner], w["norm"], u, groups=s["norm_groups"], gate_first=True, eps=eps)
-        return w["w_o"](u), None
+        return w["w_o"](u, self._f32buf(T, self.width)), None
 
     def _parallel(self, li, w, m, h, step: RaggedStep, cache: HybridCacheManager):
         T, eps = step.tokens, self.cfg.eps
         L, R = m["left"], m["right"]
         H, G, d, dv = int(L["heads"]), int(L["kv_heads"]), int(L["dim"]), int(L["vdim"])
-        qkv = w["left_qkv"](h)
+        qkv = w["left_qkv"](h, self._f32buf(T, w["left_qkv"].n))
         kc, vc = cache.k_caches[li], cache.v_caches[li]
         ops.qk_unitnorm_store(qkv, kc, vc, step, H, G, d, dv, eps)
         a = self._actbuf(T, H * dv)
         ops.window_attn(qkv, kc, vc, a, step, w["slopes"], H, G, d, dv, float(L["scale"]), int(L["mask"]["size"]))
-        left = w["left_o"](a)
+        left = w["left_o"](a, self._f32buf(T, self.width))
 
         Hr, dr, dvr, rot = int(R["heads"]), int(R["dim"]), int(R["vdim"]), int(R["rot"]["dims"])
-        qkvg = w["right_qkvg"](h)
+        qkvg = w["right_qkvg"](h, self._f32buf(T, w["right_qkvg"].n))
         q, k = qkvg[:, :Hr * dr], qkvg[:, Hr * dr:2 * Hr * dr]
         v, g = qkvg[:, 2 * Hr * dr:2 * Hr * dr + Hr * dvr], qkvg[:, 2 * Hr * dr + Hr * dvr:]
         ops.rotary_pairs_(q, w["inv_freq"], step.tok_pos, Hr, dr, rot, 1.0)
@@ -160,7 +177,7 @@ class RaggedRunner:
                        step=step, heads=Hr, n=dr, p=dvr, log_decay=w["log_decay"], chunked=self.chunked_scan)
         u = self._actbuf(T, Hr * dvr)
         ops.gated_group_norm(o, g, None, u, groups=Hr, gate_first=False, eps=eps)
-        return left, w["right_o"](u)
+        return left, w["right_o"](u, self._f32buf(T, self.width))
 
     @torch.inference_mode()
     def forward(self, step: RaggedStep, cache: HybridCacheManager, want: Optional[torch.Tensor] = None,
@@ -168,6 +185,60 @@ class RaggedRunner:
         """Run the step; returns fp32 logits [len(want), vocab] for the token indices in `want` (int32 on
         the device; None = every token).  `residuals` receives a copy of the stream after every layer
         run (debugging and tests)."""
+        if (self.use_graphs and residuals is None and step.tokens == step.rows <= self.max_graph_rows):
+            return self._replay(step, cache, want)
+        return self._run(step, cache, want, residuals)
+
+    # ------------------------------------------------------------------ captured decoding steps
+    def _replay(self, step: RaggedStep, cache: HybridCacheManager, want):
+        B = step.rows
+        entry = self._graphs.get((B, id(cache)))
+        if entry is None:
+            entry = self._capture(step, cache)
+            self._graphs[(B, id(cache))] = entry
+        graph, logits = entry[0], entry[2]
+        graph.replay()
+        if want is None:
+            return logits.clone()
+        return logits.index_select(0, want.long())
+
+    def _capture(self, step: RaggedStep, cache: HybridCacheManager):
+        """One run of the step on a side stream with fresh allocations (it sizes the arena and lets the
+        projections set up their per-stream workspaces), the recurrent state of the step's slots put back
+        as it was, then the same launches recorded over an arena.  Everything a replay reads that
+        changes from step to step - tokens, positions, slots, block table - lies in the cache manager's
+        one device buffer; keys and values of the step are written again by the replay with the same
+        contents."""
+        import ctypes
+        from ... import _native as nv
+        from .model_graph import HipGraph
+        B, slots = step.rows, list(step.slots)
+        idx = torch.tensor(slots, dtype=torch.long, device=self.device)
+        saved = [(t, t.index_select(0, idx)) for named in cache.states.values() for t in named.values()]
+        all_rows = torch.arange(B, dtype=torch.int32, device=self.device)
+        side = torch.cuda.Stream(device=self.device)
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            self._arena, self._measured = None, 0
+            self._run(step, cache, all_rows, None)
+            for t, old in saved:
+                t.index_copy_(0, idx, old)
+            arena = torch.empty(self._measured + 4096, dtype=torch.uint8, device=self.device)
+            side.synchronize()
+            self._arena, self._arena_off = arena, 0
+            nv.check("mv_graph_begin_capture", nv.lib().mv_graph_begin_capture(side.cuda_stream))
+            try:
+                logits = self._run(step, cache, all_rows, None)
+            finally:
+                handle = ctypes.c_void_p()
+                rc = nv.lib().mv_graph_end_capture(side.cuda_stream, ctypes.byref(handle))
+                self._arena = None
+            nv.check("mv_graph_end_capture", rc)
+        torch.cuda.current_stream().wait_stream(side)
+        logger.info("captured a decoding step of %d rows (%d KiB of intermediates)", B, arena.numel() >> 10)
+        return HipGraph(handle), arena, logits, all_rows      # the arena and the row list stay alive with the graph
+
+    def _run(self, step: RaggedStep, cache: HybridCacheManager, want, residuals) -> torch.Tensor:
         cfg, T = self.cfg, step.tokens
         x, h = self._f32buf(T, self.width), self._actbuf(T, self.width)
         ops.embed_scaled(self.embed, step.ids, cfg.embed_scale, x, h)
@@ -181,10 +252,10 @@ class RaggedRunner:
                 ops.postnorm_residual(y1, w["norm1"], cfg.eps, x, h, y2=y2, s1=float(m["left_scale"]),
                                       s2=float(m["right_scale"]))
             if layer.get("mlp"):
-                up = w["up"](h)
+                up = w["up"](h, self._f32buf(T, w["up"].n))
                 act = self._actbuf(T, up.shape[1])
                 ops.relu_squared(up, act)
-                ops.postnorm_residual(w["down"](act), w["norm2"], cfg.eps, x, h)
+                ops.postnorm_residual(w["down"](act, self._f32buf(T, self.width)), w["norm2"], cfg.eps, x, h)
             if residuals is not None:
                 residuals.append(x.clone())
         rows = T if want is None else want.numel()
@@ -192,7 +263,7 @@ class RaggedRunner:
         if rows == 0:
             return self._f32buf(0, self.vocab_size)
         ops.offset_rmsnorm_gather(x, want, self.final_norm, cfg.eps, normed)
-        logits = self.head(normed)
+        logits = self.head(normed, self._f32buf(rows, self.vocab_size))
         if cfg.logit_softcap:
             ops.softcap_(logits, cfg.logit_softcap)
         return logits

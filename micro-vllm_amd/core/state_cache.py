@@ -39,6 +39,7 @@ class RaggedStep:
     ch_len: torch.Tensor = None     # int32 [chunks]
     row_ch0: torch.Tensor = None    # int32 [B] the row's first chunk
     row_nch: torch.Tensor = None    # int32 [B] its number of chunks (0: a short row)
+    slots: tuple = ()               # host copy of row_slot
 
 
 SCAN_CHUNK = 64      # csrc/seq_mix.hip kCh
@@ -80,8 +81,11 @@ class HybridCacheManager:
         words = 3 * max_step_tokens + max_rows * (6 + self.max_seq_pages) + \
             2 * (max_step_tokens // SCAN_CHUNK + max_rows)
         self._ring = 4 if self._on_gpu else 1
+        # a ring of pinned staging buffers (the host may run ahead of the copies), ONE device buffer: the
+        # copies and the kernels that read it are ordered on the stream, and a step of a given shape
+        # finds its fields at the same addresses every time - what a captured step needs
         self._host = [torch.zeros(words, dtype=torch.int32, pin_memory=self._on_gpu) for _ in range(self._ring)]
-        self._dev = [torch.zeros(words, dtype=torch.int32, device=device) for _ in range(self._ring)]
+        self._dev = torch.zeros(words, dtype=torch.int32, device=device)
         self._events = [None] * self._ring
         self._next = 0
 
@@ -200,7 +204,7 @@ class HybridCacheManager:
             host[o_cs:o_cs + NC] = [c[0] for c in chunks]
             host[o_cl:o_cl + NC] = [c[1] for c in chunks]
         used = o_cl + NC
-        dev = self._dev[i]
+        dev = self._dev
         dev[:used].copy_(self._host[i][:used], non_blocking=True)
         if self._on_gpu:
             ev = self._events[i] or torch.cuda.Event()
@@ -212,4 +216,4 @@ class HybridCacheManager:
             row_ctx=dev[o_rows + 2 * B:o_rows + 3 * B], row_slot=dev[o_rows + 3 * B:o_rows + 4 * B],
             block_table=dev[o_bt:o_bt + B * W].view(B, W), max_slot=max_slot, max_page=max_page, n_chunks=NC,
             ch_start=dev[o_cs:o_cs + NC], ch_len=dev[o_cl:o_cl + NC], row_ch0=dev[o_c0:o_c0 + B],
-            row_nch=dev[o_nch:o_nch + B])
+            row_nch=dev[o_nch:o_nch + B], slots=tuple(self._slot[sid] for sid, _ in rows))

@@ -471,12 +471,13 @@ __global__ __launch_bounds__(256) void qk_unitnorm_store_kernel(float* qkv, int6
 
 constexpr int kMaxVC = 4;  // value columns per lane: vdim <= 256
 
-// One workgroup per (token, head).  Its four waves take the window's 64-key tiles in turn: a lane scores
+// One workgroup per (token, head).  Its NW waves (4, or 16 when a step has too few tokens to fill the
+// chip otherwise: decoding) take the window's 64-key tiles in turn: a lane scores
 // one key (q from LDS, the key row straight from its page), the wave forms max / sum of the tile and
 // then, lanes now owning value columns, adds the tile's weighted values; the waves' partial softmaxes
 // meet in LDS.  The same code serves a prompt's portion and a single decoded token.
-template <bool F32>
-__global__ __launch_bounds__(256) void window_attn_kernel(const float* q, int64_t ldq, const void* kc_,
+template <bool F32, int NW>
+__global__ __launch_bounds__(64 * NW) void window_attn_kernel(const float* q, int64_t ldq, const void* kc_,
                                                           const void* vc_, void* out_, int64_t ldo, PagedRows pr,
                                                           const float* slopes, int T, int H, int G, int d, int dv,
                                                           float scale, int window) {
@@ -488,18 +489,18 @@ __global__ __launch_bounds__(256) void window_attn_kernel(const float* q, int64_
     const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
     float* qs = lds;
     float* ps = lds + d + wv * 64;
-    float* mm = lds + d + 256;
-    float* ll = mm + 4;
-    float* aa = ll + 4;
+    float* mm = lds + d + 64 * NW;
+    float* ll = mm + NW;
+    float* aa = ll + NW;
     const int t = blockIdx.x / H, h = blockIdx.x % H, g = h / (H / G);
     const int pos = pr.tok_pos[t];
     const int* bt = pr.block_table + (int64_t)pr.tok_row[t] * pr.bt_stride;
     const int lo = pos - window + 1 > 0 ? pos - window + 1 : 0;
     const float slope = slopes ? slopes[h] : 0.f;
-    for (int c = threadIdx.x; c < d; c += 256) qs[c] = q[(int64_t)t * ldq + (int64_t)h * d + c];
+    for (int c = threadIdx.x; c < d; c += 64 * NW) qs[c] = q[(int64_t)t * ldq + (int64_t)h * d + c];
     __syncthreads();
     float m = -INFINITY, l = 0.f, acc[kMaxVC] = {0.f, 0.f, 0.f, 0.f};
-    for (int j0 = lo + 64 * wv; j0 <= pos; j0 += 256) {
+    for (int j0 = lo + 64 * wv; j0 <= pos; j0 += 64 * NW) {
         const int j = j0 + lane;
         float s = -INFINITY;
         if (j <= pos) {
@@ -555,10 +556,12 @@ __global__ __launch_bounds__(256) void window_attn_kernel(const float* q, int64_
     }
     __syncthreads();
     if (wv == 0) {
-        float M = fmaxf(fmaxf(mm[0], mm[1]), fmaxf(mm[2], mm[3]));   // wave 0 always has a key: finite
-        float w4[4], L = 0.f;
+        float M = mm[0];                                   // wave 0 always has a key: finite
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
+        for (int w = 1; w < NW; ++w) M = fmaxf(M, mm[w]);
+        float w4[NW], L = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
             w4[w] = expf(mm[w] - M);   // a wave without keys: exp(-inf) = 0
             L = fmaf(ll[w], w4[w], L);
         }
@@ -568,7 +571,7 @@ __global__ __launch_bounds__(256) void window_attn_kernel(const float* q, int64_
             if (c < dv) {
                 float o = 0.f;
 #pragma unroll
-                for (int w = 0; w < 4; ++w) o = fmaf(aa[w * dv + c], w4[w], o);
+                for (int w = 0; w < NW; ++w) o = fmaf(aa[w * dv + c], w4[w], o);
                 ActS<F32>::st(out + (int64_t)t * ldo + (int64_t)h * dv + c, o / L);
             }
         }
@@ -768,10 +771,19 @@ int mv_window_attn(const float* q, int64_t ldq, const void* k_cache, const void*
     const int64_t units = (int64_t)tokens * heads;
     if (units > 0x7fffffff) return MV_ERR_UNSUPPORTED;
     const dim3 grid((unsigned)units);
-    const size_t lds = (size_t)(d + 256 + 8 + 4 * dv) * sizeof(float);
     hipStream_t s = (hipStream_t)stream;
-    if (f32) hipLaunchKernelGGL(window_attn_kernel<true>, grid, dim3(256), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window);
-    else hipLaunchKernelGGL(window_attn_kernel<false>, grid, dim3(256), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window);
+    // few (token, head) pairs and a window of many tiles: sixteen waves share it
+    const bool wide = units <= 2 * num_cus() && window > 256;
+    const int nw = wide ? 16 : 4;
+    const size_t lds = (size_t)(d + 64 * nw + 2 * nw + nw * dv) * sizeof(float);
+    if (lds > 64 * 1024) return MV_ERR_UNSUPPORTED;
+    if (wide) {
+        if (f32) hipLaunchKernelGGL((window_attn_kernel<true, 16>), grid, dim3(1024), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window);
+        else hipLaunchKernelGGL((window_attn_kernel<false, 16>), grid, dim3(1024), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window);
+    } else {
+        if (f32) hipLaunchKernelGGL((window_attn_kernel<true, 4>), grid, dim3(256), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window);
+        else hipLaunchKernelGGL((window_attn_kernel<false, 4>), grid, dim3(256), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window);
+    }
     return check_launch();
 }
 

@@ -270,7 +270,8 @@ def _attend(ops, q, k, v, H, G, d, dv, scale, window, slopes, portions, f32=True
     return torch.cat(out)
 
 
-@pytest.mark.parametrize("H,G,d,dv,window", [(6, 2, 40, 56, 37), (2, 2, 64, 64, 5), (4, 1, 96, 130, 200), (3, 3, 8, 8, 1)])
+@pytest.mark.parametrize("H,G,d,dv,window", [(6, 2, 40, 56, 37), (2, 2, 64, 64, 5), (4, 1, 96, 130, 200), (3, 3, 8, 8, 1),
+                                             (2, 1, 64, 64, 300)])
 def test_window_attention_random(ops, H, G, d, dv, window):
     g = torch.Generator().manual_seed(d + window)
     T, scale = 150, 0.3
@@ -285,7 +286,7 @@ def test_window_attention_random(ops, H, G, d, dv, window):
     assert (got.double() - want).abs().max().item() < 0.05
 
 
-@pytest.mark.parametrize("window", [72, 64, 65, 130])
+@pytest.mark.parametrize("window", [72, 64, 65, 130, 260])
 @pytest.mark.parametrize("decode", [False, True])
 def test_window_edge_shows_in_the_output(ops, window, decode):
     """One key carries a value of its own and is made to win the softmax whenever it is visible: the
