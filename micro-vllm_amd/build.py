@@ -37,7 +37,7 @@ SOURCES = [
 SETS = {
     # fp32 residual stream, recurrent mixers, windowed attention; the wave-tile projections for the
     # shapes they take, and the sampler
-    "ragged": ["runtime.hip", "linear_any.hip", "stream_ops.hip", "seq_mix.hip", "wgemm.hip",
+    "ragged": ["runtime.hip", "linear_any.hip", "stream_ops.hip", "seq_mix.hip", "elementwise.hip", "wgemm.hip",
                "gemm_prefill.hip", "sampler.hip"],
 }
 
@@ -150,7 +150,8 @@ def build(force=False, verbose=True, jobs=None, only=None):
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         list(ex.map(compile_one, todo))
 
-    if force or todo or _stale(LIB, objs):
+    # a part library is linked anew every time: its list of sources may have changed since it was built
+    if force or todo or only is not None or _stale(LIB, objs):
         cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
         if verbose:
             print("[build]", " ".join(cmd), flush=True)

@@ -154,3 +154,28 @@ def test_restatement_continues_from_its_state():
     for s in range(t + 1):
         acc += decay[s + 1:t + 1, h].prod() * gain[s, h] * (q[t, h] @ k[s, h]) * v[s, h]
     assert torch.allclose(whole[t, h], acc)
+
+
+def test_part_library_holds_every_entry_point_the_family_calls(mv):
+    """The library of a part of the sources (what a first start in a fresh checkout builds) exports every
+    C entry point that the ragged family's wrappers, projections, sampler and graph capture name."""
+    import ctypes
+    import importlib.util
+    import inspect
+    import re
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("mvllm_build", os.path.join(root, "micro-vllm_amd", "build.py"))
+    b = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(b)
+    lib = b.build(verbose=False, only="ragged")
+    handle = ctypes.CDLL(lib)
+    from micro_vllm_amd.core.layer import model_graph, ragged_runner, sampler
+    from micro_vllm_amd.kernel import linear, ragged_ops
+    text = inspect.getsource(ragged_ops) + inspect.getsource(ragged_runner)
+    for fn in (linear.StreamedWeight.from_linear, linear.wgemm, linear.gemm_prefill, linear.gemm_workspace,
+               sampler.greedy, sampler.sample, model_graph.HipGraph):
+        text += inspect.getsource(fn)
+    names = {n for n in re.findall(r"\bmv_[a-z0-9_]+", text) if not n.endswith("_")} | {"mv_status_string", "mv_last_hip_error", "mv_version"}
+    assert {"mv_shuffle_weight", "mv_scan_chunked", "mv_graph_launch", "mv_wgemm"} <= names
+    missing = sorted(n for n in names if not hasattr(handle, n))
+    assert not missing, missing
