@@ -658,6 +658,8 @@ int mv_scan_outer(const float* q, int64_t ldq, int q_div, const float* k, int64_
     a.r = StepRows{nullptr, nullptr, row_start, row_len, row_ctx, row_slot};
     a.H = heads; a.n = n; a.p = p; a.max_len = max_len;
     a.pt = p % 64 == 0 ? 64 : (p % 32 == 0 ? 32 : 16);
+    // a state too tall for 64 rows a thread: narrower column tiles leave more threads to share its rows
+    while (a.pt > 16 && (n + 256 / a.pt - 1) / (256 / a.pt) > 64) a.pt /= 2;
     const int ns = 256 / a.pt, npt = (n + ns - 1) / ns;
     const dim3 grid((p + a.pt - 1) / a.pt, heads, rows);
     hipStream_t s = (hipStream_t)stream;
