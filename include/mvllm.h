@@ -549,11 +549,17 @@ int mv_qk_unitnorm_store(float* qkv, int64_t ld, void* k_cache, void* v_cache, c
                          int heads, int kv_heads, int d, int dv, float eps, int f32, mv_stream_t stream);
 
 /* out[t, h*dv ..] = softmax_j( q_t . k_j * scale - slopes[h] * (pos - j) ) v_j over pos - window < j <= pos
- * from the pages (the step's own keys must already be stored).  dv <= 256. */
+ * from the pages (the step's own keys must already be stored).  dv <= 256.  With a chunk table (chunks > 0:
+ * rows of more than max_len tokens cut into runs of up to 64, as for mv_scan_chunked; row_len per row), bf16
+ * and a head shape the tiled kernel is built for - (d, dv) in (32,32) (64,64) (96,96) (128,128) (128,64)
+ * (64,128), 64-token pages - those rows run on the matrix cores, a workgroup per (chunk, head): q.k in bf16
+ * (q rounded as the cached keys are), softmax in fp32, P.V with fp32 P.  Every other token takes the
+ * one-workgroup-per-(token, head) form. */
 int mv_window_attn(const float* q, int64_t ldq, const void* k_cache, const void* v_cache, void* out, int64_t ldo,
                    const int32_t* tok_row, const int32_t* tok_pos, const int32_t* block_table, int bt_stride,
                    int page, const float* slopes, int tokens, int heads, int kv_heads, int d, int dv, float scale,
-                   int window, int f32, mv_stream_t stream);
+                   int window, int f32, const int32_t* row_len, const int32_t* ch_start, const int32_t* ch_len,
+                   int chunks, int max_len, mv_stream_t stream);
 
 #ifdef __cplusplus
 }

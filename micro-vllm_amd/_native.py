@@ -107,7 +107,8 @@ PROTOTYPES = {
     "mv_rotary_pairs": (_I, [_P, _L, _P, _P, _I, _I, _I, _I, _F, _P]),
     "mv_gated_group_norm": (_I, [_P, _L, _P, _L, _P, _P, _L, _I, _I, _I, _I, _F, _I, _P]),
     "mv_qk_unitnorm_store": (_I, [_P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P]),
-    "mv_window_attn": (_I, [_P, _L, _P, _P, _P, _L, _P, _P, _P, _I, _I, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P]),
+    "mv_window_attn": (_I, [_P, _L, _P, _P, _P, _L, _P, _P, _P, _I, _I, _P, _I, _I, _I, _I, _I, _F, _I, _I,
+                            _P, _P, _P, _I, _I, _P]),
     "mv_graph_begin_capture": (_I, [_P]),
     "mv_graph_end_capture": (_I, [_P, ctypes.POINTER(c_void_p)]),
     "mv_graph_launch": (_I, [_P, _P]),

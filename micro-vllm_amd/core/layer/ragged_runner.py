@@ -34,13 +34,14 @@ class RaggedRunner:
     PAGE = 64
 
     def __init__(self, model, device="cuda", dtype=torch.bfloat16, wave_tiles: bool = True,
-                 chunked_scan: bool = True, graphs: bool = True, max_graph_rows: int = 64):
+                 chunked_scan: bool = True, graphs: bool = True, max_graph_rows: int = 64, tiled_attn: bool = True):
         """`wave_tiles` / `chunked_scan` = False keep every projection on the plain any-shape kernel and
-        every recurrence token by token (the forms the faster ones are checked against).  `graphs`:
+        every recurrence token by token, `tiled_attn` = False every token on the plain attention kernel (the
+        forms the faster ones are checked against).  `graphs`:
         steps in which every row brings one token (decoding) are captured once per row count into a
         hipGraph and replayed - some seventy launches become one."""
         assert dtype in (torch.bfloat16, torch.float32)
-        self.chunked_scan = chunked_scan
+        self.chunked_scan, self.tiled_attn = chunked_scan, tiled_attn
         self.use_graphs, self.max_graph_rows = graphs, max_graph_rows
         self._graphs: Dict[int, tuple] = {}
         self._arena, self._arena_off, self._measured = None, 0, 0
@@ -163,7 +164,8 @@ class RaggedRunner:
         kc, vc = cache.k_caches[li], cache.v_caches[li]
         ops.qk_unitnorm_store(qkv, kc, vc, step, H, G, d, dv, eps)
         a = self._actbuf(T, H * dv)
-        ops.window_attn(qkv, kc, vc, a, step, w["slopes"], H, G, d, dv, float(L["scale"]), int(L["mask"]["size"]))
+        ops.window_attn(qkv, kc, vc, a, step, w["slopes"], H, G, d, dv, float(L["scale"]), int(L["mask"]["size"]),
+                        tiled=self.tiled_attn)
         left = w["left_o"](a, self._f32buf(T, self.width))
 
         Hr, dr, dvr, rot = int(R["heads"]), int(R["dim"]), int(R["vdim"]), int(R["rot"]["dims"])

@@ -42,8 +42,9 @@ class RaggedStep:
     slots: tuple = ()               # host copy of row_slot
 
 
+from ..kernel.ragged_ops import SCAN_SEQ_MAX  # noqa: E402  rows up to this length are not cut into chunks
+
 SCAN_CHUNK = 64      # csrc/seq_mix.hip kCh
-SCAN_SEQ_MAX = 16    # rows up to this length run the recurrence token by token
 
 
 class PoolExhausted(RuntimeError):

@@ -480,9 +480,10 @@ template <bool F32, int NW>
 __global__ __launch_bounds__(64 * NW) void window_attn_kernel(const float* q, int64_t ldq, const void* kc_,
                                                           const void* vc_, void* out_, int64_t ldo, PagedRows pr,
                                                           const float* slopes, int T, int H, int G, int d, int dv,
-                                                          float scale, int window) {
+                                                          float scale, int window, const int* row_len, int max_len) {
     typedef typename ActS<F32>::T T_;
     extern __shared__ float lds[];
+    if (max_len > 0 && row_len[pr.tok_row[blockIdx.x / H]] > max_len) return;   // the tiled kernel's rows
     const T_* kc = (const T_*)kc_;
     const T_* vc = (const T_*)vc_;
     T_* out = (T_*)out_;
@@ -574,6 +575,127 @@ __global__ __launch_bounds__(64 * NW) void window_attn_kernel(const float* q, in
                 for (int w = 0; w < NW; ++w) o = fmaf(aa[w * dv + c], w4[w], o);
                 ActS<F32>::st(out + (int64_t)t * ldo + (int64_t)h * dv + c, o / L);
             }
+        }
+    }
+}
+
+// The same attention for a prompt's portion, bf16 keys and values: one workgroup per (64 consecutive tokens
+// of a row, head).  Key tiles are pages (64 tokens) staged once in LDS for all 64 queries; q.k on
+// v_mfma_f32_16x16x32_bf16 (q rounded to bf16 as the keys are), scores, distance penalty, mask and softmax
+// in fp32 per lane, and P.V on v_mfma_f32_16x16x4_f32 with P staying fp32: the score accumulators of a lane,
+// S[key 16 nt + 4 (lane / 16) + j][query lane % 16], are exactly the second operand of that instruction
+// for the four keys {16 nt + j + 4 k}, so P never leaves the registers.
+typedef __attribute__((ext_vector_type(8))) __bf16 wa_bf16x8_t;
+
+template <int KS, int CT>
+__global__ __launch_bounds__(256) void window_attn_tile_kernel(const float* q, int64_t ldq, const uint16_t* kc,
+                                                               const uint16_t* vc, uint16_t* out, int64_t ldo,
+                                                               PagedRows pr, const int* ch_start, const int* ch_len,
+                                                               const float* slopes, int H, int G, float scale,
+                                                               int window) {
+    constexpr int D = KS * 32, DV = CT * 16, SK = D + 8, SV = DV + 8;
+    __shared__ __attribute__((aligned(16))) uint16_t Ks[64][SK];
+    __shared__ __attribute__((aligned(16))) uint16_t Vs[64][SV];
+    const int ch = blockIdx.x, h = blockIdx.y, g = h / (H / G);
+    const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, r = lane & 15, qd = lane >> 4;
+    const int start = ch_start[ch], len = ch_len[ch];
+    const int* bt = pr.block_table + (int64_t)pr.tok_row[start] * pr.bt_stride;
+    const int p0 = pr.tok_pos[start];            // positions run on from here within the chunk
+    const int myq = 16 * wv + r;
+    const bool qok = myq < len;
+    const int qpos = p0 + myq;
+    wa_bf16x8_t qf[KS];
+    {
+        const float* qp = q + (int64_t)(start + (qok ? myq : 0)) * ldq + (int64_t)h * D + 8 * qd;
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) {
+            const float4 a = *reinterpret_cast<const float4*>(qp + 32 * kk);
+            const float4 b = *reinterpret_cast<const float4*>(qp + 32 * kk + 4);
+            const uint4 pk = make_uint4(pack_bf16x2(a.x, a.y), pack_bf16x2(a.z, a.w), pack_bf16x2(b.x, b.y),
+                                        pack_bf16x2(b.z, b.w));
+            qf[kk] = __builtin_bit_cast(wa_bf16x8_t, pk);
+        }
+    }
+    float m = -INFINITY, l = 0.f;
+    f32x4_t o[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) o[ct] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    const float slope = slopes ? slopes[h] : 0.f;
+    const int klo = p0 - window + 1 > 0 ? p0 - window + 1 : 0, khi = p0 + len - 1;
+    const int wq_lo = p0 + 16 * wv, wq_hi = wq_lo + 15;   // this wave's query positions
+    for (int kt = klo / 64; kt <= khi / 64; ++kt) {
+        const int kbase = kt * 64;
+        const int64_t pgrow = (int64_t)bt[kt] * 64;
+        __syncthreads();
+        for (int i = tid; i < 64 * (D / 8); i += 256) {
+            const int rr = i / (D / 8), cc = i % (D / 8);
+            st16(&Ks[rr][cc * 8], ld16(kc + ((pgrow + rr) * G + g) * D + cc * 8));
+        }
+        for (int i = tid; i < 64 * (DV / 8); i += 256) {
+            const int rr = i / (DV / 8), cc = i % (DV / 8);
+            st16(&Vs[rr][cc * 8], ld16(vc + ((pgrow + rr) * G + g) * DV + cc * 8));
+        }
+        __syncthreads();
+        if (kbase > wq_hi || kbase + 63 <= wq_lo - window) continue;   // nothing of this tile is visible to the wave
+        f32x4_t sc[4];
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) {
+            sc[nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kk = 0; kk < KS; ++kk) {
+                const wa_bf16x8_t kf = __builtin_bit_cast(wa_bf16x8_t, ld16(&Ks[16 * nt + r][32 * kk + 8 * qd]));
+                sc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[kk], sc[nt], 0, 0, 0);
+            }
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int kpos = kbase + 16 * nt + 4 * qd + j;
+                const bool ok = qok && kpos <= qpos && kpos > qpos - window;
+                const float v = ok ? sc[nt][j] * scale - slope * (float)(qpos - kpos) : -INFINITY;
+                sc[nt][j] = v;
+                mx = fmaxf(mx, v);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float mn = fmaxf(m, mx);
+        const float corr = m == -INFINITY ? 0.f : expf(m - mn);
+        float ps = 0.f;
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float pv = sc[nt][j] == -INFINITY ? 0.f : expf(sc[nt][j] - mn);
+                sc[nt][j] = pv;
+                ps += pv;
+            }
+        ps += __shfl_xor(ps, 16, 64);
+        ps += __shfl_xor(ps, 32, 64);
+        l = l * corr + ps;
+        m = mn;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) o[ct] *= corr;
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint16_t* vrow = &Vs[16 * nt + 4 * qd + j][r];
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct)
+                    o[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(bf16_bits_to_f32(vrow[16 * ct]), sc[nt][j], o[ct], 0, 0, 0);
+            }
+    }
+    if (qok) {
+        const float inv = 1.0f / l;
+        uint16_t* op = out + (int64_t)(start + myq) * ldo + (int64_t)h * DV + 4 * qd;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            uint2 w;
+            w.x = pack_bf16x2(o[ct][0] * inv, o[ct][1] * inv);
+            w.y = pack_bf16x2(o[ct][2] * inv, o[ct][3] * inv);
+            *reinterpret_cast<uint2*>(op + 16 * ct) = w;
         }
     }
 }
@@ -761,7 +883,8 @@ int mv_qk_unitnorm_store(float* qkv, int64_t ld, void* k_cache, void* v_cache, c
 int mv_window_attn(const float* q, int64_t ldq, const void* k_cache, const void* v_cache, void* out, int64_t ldo,
                    const int32_t* tok_row, const int32_t* tok_pos, const int32_t* block_table, int bt_stride,
                    int page, const float* slopes, int tokens, int heads, int kv_heads, int d, int dv, float scale,
-                   int window, int f32, mv_stream_t stream) {
+                   int window, int f32, const int32_t* row_len, const int32_t* ch_start, const int32_t* ch_len,
+                   int chunks, int max_len, mv_stream_t stream) {
     using namespace mv;
     if (tokens < 0 || heads <= 0 || kv_heads <= 0 || d <= 0 || dv <= 0 || page <= 0 || window <= 0 ||
         heads % kv_heads)
@@ -774,17 +897,36 @@ int mv_window_attn(const float* q, int64_t ldq, const void* k_cache, const void*
     if (units > 0x7fffffff) return MV_ERR_UNSUPPORTED;
     const dim3 grid((unsigned)units);
     hipStream_t s = (hipStream_t)stream;
+    // rows of more than max_len tokens, cut into the chunks of the table: the tiled matrix-core kernel, where
+    // the shapes are among those it is built for (bf16, 64-token pages, 16-byte rows)
+    int skip_len = 0;
+    if (!f32 && chunks > 0 && max_len > 0 && row_len && ch_start && ch_len && page == 64 && ldq % 4 == 0 &&
+        ldo % 4 == 0 && aligned16(q) && aligned16(k_cache) && aligned16(v_cache) && (reinterpret_cast<uintptr_t>(out) & 7) == 0) {
+        const dim3 tg(chunks, heads);
+#define MV_WA_TILE(KS_, CT_)                                                                                         \
+    hipLaunchKernelGGL((window_attn_tile_kernel<KS_, CT_>), tg, dim3(256), 0, s, q, ldq, (const uint16_t*)k_cache,      \
+                       (const uint16_t*)v_cache, (uint16_t*)out, ldo, pr, ch_start, ch_len, slopes, heads, kv_heads, scale, \
+                       window);                                                                                       \
+    skip_len = max_len
+        if (d == 64 && dv == 64) { MV_WA_TILE(2, 4); }
+        else if (d == 96 && dv == 96) { MV_WA_TILE(3, 6); }
+        else if (d == 128 && dv == 128) { MV_WA_TILE(4, 8); }
+        else if (d == 128 && dv == 64) { MV_WA_TILE(4, 4); }
+        else if (d == 64 && dv == 128) { MV_WA_TILE(2, 8); }
+        else if (d == 32 && dv == 32) { MV_WA_TILE(1, 2); }
+#undef MV_WA_TILE
+    }
     // few (token, head) pairs and a window of many tiles: sixteen waves share it
     const bool wide = units <= 2 * num_cus() && window > 256;
     const int nw = wide ? 16 : 4;
     const size_t lds = (size_t)(d + 64 * nw + 2 * nw + nw * dv) * sizeof(float);
     if (lds > 64 * 1024) return MV_ERR_UNSUPPORTED;
     if (wide) {
-        if (f32) hipLaunchKernelGGL((window_attn_kernel<true, 16>), grid, dim3(1024), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window);
-        else hipLaunchKernelGGL((window_attn_kernel<false, 16>), grid, dim3(1024), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window);
+        if (f32) hipLaunchKernelGGL((window_attn_kernel<true, 16>), grid, dim3(1024), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window, row_len, skip_len);
+        else hipLaunchKernelGGL((window_attn_kernel<false, 16>), grid, dim3(1024), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window, row_len, skip_len);
     } else {
-        if (f32) hipLaunchKernelGGL((window_attn_kernel<true, 4>), grid, dim3(256), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window);
-        else hipLaunchKernelGGL((window_attn_kernel<false, 4>), grid, dim3(256), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window);
+        if (f32) hipLaunchKernelGGL((window_attn_kernel<true, 4>), grid, dim3(256), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window, row_len, skip_len);
+        else hipLaunchKernelGGL((window_attn_kernel<false, 4>), grid, dim3(256), lds, s, q, ldq, k_cache, v_cache, out, ldo, pr, slopes, tokens, heads, kv_heads, d, dv, scale, window, row_len, skip_len);
     }
     return check_launch();
 }

@@ -13,6 +13,9 @@ import torch
 from .. import _native as nv
 from .linear import StreamedWeight, gemm_prefill, wgemm
 
+SCAN_SEQ_MAX = 16   # rows up to this length are not in a step's chunk table (core/state_cache.py): they take the
+                    # token-by-token recurrence and the one-workgroup-per-token attention
+
 
 def _ld(t: torch.Tensor) -> int:
     assert t.dim() == 2 and t.stride(1) == 1
@@ -177,7 +180,6 @@ def scan_outer(q, k, v, decay, gain, skip, state, out, step, heads: int, n: int,
             ds.data_ptr(), lsum.data_ptr(), atot.data_ptr(), step.ch_start.data_ptr(), step.ch_len.data_ptr(),
             step.row_ch0.data_ptr(), step.row_nch.data_ptr(), step.row_ctx.data_ptr(), step.row_slot.data_ptr(),
             step.n_chunks, step.rows, heads, n, p, nv.stream_ptr()))
-    from ..core.state_cache import SCAN_SEQ_MAX
     nv.check("mv_scan_outer", nv.lib().mv_scan_outer(
         _f32(q).data_ptr(), _ld(q), q_div, _f32(k).data_ptr(), _ld(k), k_div, _f32(v).data_ptr(), _ld(v),
         _f32(decay).data_ptr(), ld_decay, None if gain is None else _f32(gain).data_ptr(),
@@ -219,7 +221,9 @@ def qk_unitnorm_store(qkv, k_cache, v_cache, step, heads: int, kv_heads: int, d:
 
 
 def window_attn(q, k_cache, v_cache, out, step, slopes, heads: int, kv_heads: int, d: int, dv: int,
-                scale: float, window: int):
+                scale: float, window: int, tiled: bool = True):
+    """`tiled`: rows of more than SCAN_SEQ_MAX tokens go to the matrix-core kernel where it applies (bf16,
+    the head shapes it is built for); False keeps every token on the plain kernel."""
     tokens = q.shape[0]
     assert q.shape[1] >= heads * d and out.shape == (tokens, heads * dv) and out.dtype == k_cache.dtype
     page = k_cache.shape[1]
@@ -230,4 +234,6 @@ def window_attn(q, k_cache, v_cache, out, step, slopes, heads: int, kv_heads: in
         _f32(q).data_ptr(), _ld(q), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _ld(out),
         step.tok_row.data_ptr(), step.tok_pos.data_ptr(), step.block_table.data_ptr(), step.block_table.stride(0),
         page, None if slopes is None else _f32(slopes).data_ptr(), tokens, heads, kv_heads, d, dv, float(scale),
-        int(window), _is_f32(k_cache), nv.stream_ptr()))
+        int(window), _is_f32(k_cache), step.row_len.data_ptr(),
+        step.ch_start.data_ptr() if step.n_chunks else None, step.ch_len.data_ptr() if step.n_chunks else None,
+        step.n_chunks if tiled else 0, SCAN_SEQ_MAX, nv.stream_ptr()))

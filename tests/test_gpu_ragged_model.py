@@ -61,16 +61,17 @@ def test_portions_and_decoding_match_the_whole_prompt_fp32(make):
 
 
 def test_token_by_token_forms_agree_with_the_fast_ones():
-    """The plain any-shape projection and the token-by-token recurrence against the wave-tile projections
-    and the chunked recurrence the runner takes by default."""
+    """The plain any-shape projection, the token-by-token recurrence, the one-workgroup-per-token attention and
+    uncaptured decoding steps against the forms the runner takes by default."""
     from micro_vllm_amd.core.layer.ragged_runner import RaggedRunner
     cfg = config_b()
     toks = tokens_for(cfg, 200, 15)
     for dtype, tol in ((torch.float32, 2e-5), (torch.bfloat16, 2e-2)):
         eng = make_engine(cfg, dtype)
-        fast = run_in_portions(eng, "f", toks, [130, 70])
-        eng.runner = RaggedRunner(eng.model, eng.device, dtype, wave_tiles=False, chunked_scan=False)
-        slow = run_in_portions(eng, "s", toks, [130, 70])
+        fast = run_in_portions(eng, "f", toks, [130, 50] + [1] * 20)
+        eng.runner = RaggedRunner(eng.model, eng.device, dtype, wave_tiles=False, chunked_scan=False, tiled_attn=False,
+                                  graphs=False)
+        slow = run_in_portions(eng, "s", toks, [130, 50] + [1] * 20)
         assert rel_err(fast, slow) < tol
 
 

@@ -244,7 +244,7 @@ def test_gated_group_norm_both_orders(ops, f32):
         assert (out.cpu().double() - want).abs().max().item() < tol * max(1.0, want.abs().max().item())
 
 
-def _attend(ops, q, k, v, H, G, d, dv, scale, window, slopes, portions, f32=True, pages=16, shuffle=True):
+def _attend(ops, q, k, v, H, G, d, dv, scale, window, slopes, portions, f32=True, pages=16, shuffle=True, tiled=True):
     """Feed q|k|v rows in portions through qk_unitnorm_store + window_attn; returns [T, H*dv]."""
     dt = torch.float32 if f32 else torch.bfloat16
     cache = make_cache(kv={0: (G, d, dv)}, pages=pages, dtype=dt, max_tokens=pages * 64)
@@ -264,7 +264,7 @@ def _attend(ops, q, k, v, H, G, d, dv, scale, window, slopes, portions, f32=True
         ops.qk_unitnorm_store(rows, cache.k_caches[0], cache.v_caches[0], st, H, G, d, dv, 1e-6)
         o = torch.empty(n, H * dv, dtype=dt, device=DEV)
         ops.window_attn(rows, cache.k_caches[0], cache.v_caches[0], o, st, torch.tensor(slopes).float().to(DEV), H, G, d,
-                        dv, scale, window)
+                        dv, scale, window, tiled=tiled)
         out.append(o.float().cpu())
         pos += n
     return torch.cat(out)
@@ -282,17 +282,36 @@ def test_window_attention_random(ops, H, G, d, dv, window):
     for portions in ([T], [64, 64, 22], [3, 61, 2, 63, 1, 20], [100] + [1] * 50):
         got = _attend(ops, q, k, v, H, G, d, dv, scale, window, slopes, portions)
         assert (got.double() - want).abs().max().item() < 1e-4, portions
-    got = _attend(ops, q, k, v, H, G, d, dv, scale, window, slopes, [T], f32=False)
+    got = _attend(ops, q, k, v, H, G, d, dv, scale, window, slopes, [T], f32=False, tiled=False)
     assert (got.double() - want).abs().max().item() < 0.05
 
 
+@pytest.mark.parametrize("H,G,d,dv,window", [(2, 2, 64, 64, 5), (4, 2, 128, 64, 100), (3, 1, 96, 96, 72), (2, 1, 32, 32, 40),
+                                             (8, 2, 128, 128, 64), (2, 2, 64, 128, 300)])
+def test_window_attention_on_the_matrix_cores(ops, H, G, d, dv, window):
+    """Long rows in bf16: the tiled kernel against the restatement and against the plain kernel, whole and
+    in portions that start in the middle of a page, a short row riding along on the plain kernel."""
+    g = torch.Generator().manual_seed(d * 3 + window)
+    T, scale = 333, 0.3
+    q, k, v = torch.randn(T, H, d, generator=g), torch.randn(T, G, d, generator=g), torch.randn(T, G, dv, generator=g)
+    slopes = [2.0 ** (-8.0 * (h + 1) / H) for h in range(H)]
+    want = ref.windowed_softmax_attention(ref.unit_rms(q.double(), 1e-6), ref.unit_rms(k.double(), 1e-6), v.double(),
+                                          scale, window, slopes).reshape(T, H * dv)
+    plain = _attend(ops, q, k, v, H, G, d, dv, scale, window, slopes, [T], f32=False, tiled=False)
+    for portions in ([T], [70, 3, 129, 17, 64, 50], [200] + [1] * 133):
+        got = _attend(ops, q, k, v, H, G, d, dv, scale, window, slopes, portions, f32=False)
+        assert (got.double() - want).abs().max().item() < 0.06, portions
+        assert (got - plain).abs().max().item() < 0.06, portions
+    assert (got.double() - want).abs().mean().item() < 0.006
+
+
 @pytest.mark.parametrize("window", [72, 64, 65, 130, 260])
-@pytest.mark.parametrize("decode", [False, True])
-def test_window_edge_shows_in_the_output(ops, window, decode):
+@pytest.mark.parametrize("decode,f32", [(False, True), (True, True), (False, False)])
+def test_window_edge_shows_in_the_output(ops, window, decode, f32):
     """One key carries a value of its own and is made to win the softmax whenever it is visible: the
     query that still sees it (distance window - 1) returns that value, the next one does not."""
     H = G = 1
-    d = dv = 16
+    d = dv = 32              # a head shape the tiled bf16 kernel takes, so the bf16 prompt run goes through it
     T = 2 * window + 70
     g = torch.Generator().manual_seed(window)
     q, k, v = torch.randn(T, H, d, generator=g) * 0.01, torch.randn(T, G, d, generator=g) * 0.01, torch.zeros(T, G, dv)
@@ -308,9 +327,9 @@ def test_window_edge_shows_in_the_output(ops, window, decode):
         for i in (mark + window - 1, mark + window):     # just inside, just outside
             qq[i, 0] = 0
             qq[i, 0, n] = 1.0
-        out = _attend(ops, qq, k, v, H, G, d, dv, 40.0, window, [0.0], portions)
+        out = _attend(ops, qq, k, v, H, G, d, dv, 40.0, window, [0.0], portions, f32=f32)
         seen[mark] = (out[mark + window - 1, 0].item(), out[mark + window, 0].item())
-        assert abs(seen[mark][0] - (100.0 + mark)) < 1.0, (mark, seen)
+        assert abs(seen[mark][0] - (100.0 + mark)) < (1.0 if f32 else 2.5), (mark, seen)
         assert abs(seen[mark][1]) < 60.0 and abs(seen[mark][1] - (100.0 + mark)) > 40.0, (mark, seen)
 
 
