@@ -513,8 +513,9 @@ int mv_scan_outer(const float* q, int64_t ldq, int q_div, const float* k, int64_
                   const int32_t* row_len, const int32_t* row_ctx, const int32_t* row_slot, int rows, int heads, int n,
                   int p, int max_len, mv_stream_t stream);
 
-/* The same recurrence for long rows, 64 tokens at a time (three launches: sums within each chunk, the
- * states the chunks start from, their contribution to the outputs).  Chunk c covers tokens ch_start[c] ..
+/* The same recurrence for long rows, 64 tokens at a time, its products on the fp32 matrix instruction
+ * (v_mfma_f32_16x16x4_f32; three launches: sums within each chunk, the states the chunks start from, their
+ * contribution to the outputs).  Chunk c covers tokens ch_start[c] ..
  * + ch_len[c] (<= 64) of one row; row b owns chunks row_ch0[b] .. + row_nch[b] (0: the row is not taken -
  * mv_scan_outer with max_len > 0 leaves exactly the rows longer than max_len to this call).  The decay
  * comes as its logarithm ([tokens, heads], or [heads] with ld_ld == 0).  Scratch: ds [chunks, heads, n, p],

@@ -177,20 +177,24 @@ struct ChunkArgs {
     int H, n, p;
 };
 
+// All three products of a chunk run on v_mfma_f32_16x16x4_f32 (true fp32): operand A lane (r, g) = A[r][g],
+// operand B lane (r, g) = B[g][r], result lane (r, g) = C[4 g + j][r] (r = lane % 16, g = lane / 16).
+#define MV_MFMA4(acc, a_, b_) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a_, b_, acc, 0, 0, 0)
+
 __global__ __launch_bounds__(256) void scan_chunk_intra_kernel(ChunkArgs a) {
     extern __shared__ float lds[];
     const int ch = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
-    const int n = a.n, p = a.p, sn = n + 1, sp = p + 1, sc = kCh + 1;
+    const int wv = tid >> 6, r = tid & 15, qd = (tid & 63) >> 4;
+    const int n = a.n, p = a.p, n4 = (n + 3) & ~3, sn = n4 + 1, sp = p + 1;
     float* qs = lds;
     float* ks = qs + kCh * sn;
     float* vs = ks + kCh * sn;
-    float* ps = vs + kCh * sp;
-    float* Ls = ps + kCh * sc;
+    float* Ls = vs + kCh * sp;
     float* gs = Ls + kCh;
     const int start = a.ch_start[ch], len = a.ch_len[ch];
-    for (int i = tid; i < kCh * n; i += 256) {
-        const int t = i / n, j = i % n;
-        const bool ok = t < len;
+    for (int i = tid; i < kCh * n4; i += 256) {
+        const int t = i / n4, j = i % n4;
+        const bool ok = t < len && j < n;
         qs[t * sn + j] = ok ? a.q[(int64_t)(start + t) * a.ldq + (int64_t)(h / a.q_div) * n + j] : 0.f;
         ks[t * sn + j] = ok ? a.k[(int64_t)(start + t) * a.ldk + (int64_t)(h / a.k_div) * n + j] : 0.f;
     }
@@ -216,100 +220,86 @@ __global__ __launch_bounds__(256) void scan_chunk_intra_kernel(ChunkArgs a) {
     __syncthreads();
     const float Lend = Ls[len - 1];
     if (tid == 0) a.atot[(int64_t)ch * a.H + h] = expf(Lend);
-    const int tt = tid >> 4, cc = tid & 15;
-    // P[t][s] = (q_t . k_s) exp(L_t - L_s) gain_s for s <= t: 4 x 4 entries per thread
+    // wave wv owns the tokens t = 16 wv + r.  P[nt][j] = P[t][s = 16 nt + 4 qd + j], s-tiles above the diagonal
+    // stay zero: A = k rows of the s-tile, B = q rows of the wave's tokens, summed over the state index
+    const int t0 = 16 * wv, t = t0 + r;
+    f32x4_t P[4];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) P[nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int j0 = 0; j0 < n4; j0 += 4) {
+        const float bq = qs[t * sn + j0 + qd];
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+            if (nt <= wv) MV_MFMA4(P[nt], ks[(16 * nt + r) * sn + j0 + qd], bq);
+    }
     {
-        const int t0 = tt * 4, s0 = cc * 4;
-        float acc[4][4] = {};
-        if (s0 <= t0 + 3) {
-            for (int j = 0; j < n; ++j) {
-                float qv[4], kv[4];
+        const float Lt = Ls[t];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    qv[i] = qs[(t0 + i) * sn + j];
-                    kv[i] = ks[(s0 + i) * sn + j];
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int s_ = 16 * nt + 4 * qd + j;
+                P[nt][j] = (s_ <= t) ? P[nt][j] * expf(Lt - Ls[s_]) * gs[s_] : 0.f;
+            }
+    }
+    // o[t][c] = sum_s P[t][s] v[s][c]: A = v^T (columns c), B = P straight from the registers
+    for (int c0 = 0; c0 < p; c0 += 64) {
+        f32x4_t o[4];
+#pragma unroll
+        for (int ct = 0; ct < 4; ++ct) o[ct] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) {
+            if (nt > wv) continue;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float* vrow = vs + (16 * nt + 4 * qd + j) * sp;
+#pragma unroll
+                for (int ct = 0; ct < 4; ++ct) {
+                    const int c = c0 + 16 * ct + r;
+                    MV_MFMA4(o[ct], c < p ? vrow[c] : 0.f, P[nt][j]);
                 }
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) acc[i][e] = fmaf(qv[i], kv[e], acc[i][e]);
             }
         }
+        if (t < len) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+            for (int ct = 0; ct < 4; ++ct)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int t = t0 + i, s_ = s0 + e;
-                ps[t * sc + s_] = (s_ <= t) ? acc[i][e] * expf(Ls[t] - Ls[s_]) * gs[s_] : 0.f;
-            }
-    }
-    __syncthreads();
-    // o[t][c] = sum_s P[t][s] v[s][c]: rows 4 tt .. + 3, columns cc + 16 i
-    for (int c0 = 0; c0 < p; c0 += 128) {
-        float acc[4][8] = {};
-        for (int s_ = 0; s_ < kCh; ++s_) {
-            float pv[4], vv[8];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) pv[i] = ps[(tt * 4 + i) * sc + s_];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int c = c0 + cc + 16 * e;
-                vv[e] = c < p ? vs[s_ * sp + c] : 0.f;
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int e = 0; e < 8; ++e) acc[i][e] = fmaf(pv[i], vv[e], acc[i][e]);
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int t = tt * 4 + i;
-            if (t >= len) continue;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int c = c0 + cc + 16 * e;
-                if (c < p) a.out[(int64_t)(start + t) * a.ldo + (int64_t)h * p + c] = acc[i][e];
-            }
+                for (int j = 0; j < 4; ++j) {
+                    const int c = c0 + 16 * ct + 4 * qd + j;
+                    if (c < p) a.out[(int64_t)(start + t) * a.ldo + (int64_t)h * p + c] = o[ct][j];
+                }
         }
     }
-    // k_s <- k_s exp(L_end - L_s) gain_s, then dS[j][c] = sum_s k[s][j] v[s][c]
+    // k_s <- k_s exp(L_end - L_s) gain_s, then dS[j][c] = sum_s k[s][j] v[s][c]: A = k^T, B = v, over the tokens
     __syncthreads();
-    for (int i = tid; i < kCh * n; i += 256) {
-        const int t = i / n, j = i % n;
-        ks[t * sn + j] *= expf(Lend - Ls[t]) * gs[t];
+    for (int i = tid; i < kCh * n4; i += 256) {
+        const int tt = i / n4, j = i % n4;
+        ks[tt * sn + j] *= expf(Lend - Ls[tt]) * gs[tt];
     }
     __syncthreads();
     float* dsp = a.ds + ((int64_t)ch * a.H + h) * n * p;
-    for (int j0 = 0; j0 < n; j0 += 64) {
-        for (int c0 = 0; c0 < p; c0 += 128) {
-            float acc[4][8] = {};
-            for (int s_ = 0; s_ < len; ++s_) {
-                float kv[4], vv[8];
+    for (int jt = wv; jt * 16 < n; jt += 4) {
+        const int ja = 16 * jt + r;
+        for (int c0 = 0; c0 < p; c0 += 64) {
+            f32x4_t dd[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int j = j0 + tt + 16 * i;
-                    kv[i] = j < n ? ks[s_ * sn + j] : 0.f;
-                }
+            for (int ct = 0; ct < 4; ++ct) dd[ct] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            for (int s0 = 0; s0 < kCh; s0 += 4) {
+                const float ak = ja < n4 ? ks[(s0 + qd) * sn + ja] : 0.f;
+                const float* vrow = vs + (s0 + qd) * sp;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const int c = c0 + cc + 16 * e;
-                    vv[e] = c < p ? vs[s_ * sp + c] : 0.f;
-                }
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) acc[i][e] = fmaf(kv[i], vv[e], acc[i][e]);
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int j = j0 + tt + 16 * i;
-                if (j >= n) continue;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const int c = c0 + cc + 16 * e;
-                    if (c < p) dsp[(int64_t)j * p + c] = acc[i][e];
+                for (int ct = 0; ct < 4; ++ct) {
+                    const int c = c0 + 16 * ct + r;
+                    MV_MFMA4(dd[ct], ak, c < p ? vrow[c] : 0.f);
                 }
             }
+#pragma unroll
+            for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int jj = 16 * jt + 4 * qd + j, c = c0 + 16 * ct + r;
+                    if (jj < n && c < p) dsp[(int64_t)jj * p + c] = dd[ct][j];
+                }
         }
     }
 }
@@ -334,49 +324,47 @@ __global__ __launch_bounds__(256) void scan_chunk_carry_kernel(ChunkArgs a) {
 __global__ __launch_bounds__(256) void scan_chunk_inter_kernel(ChunkArgs a) {
     extern __shared__ float lds[];
     const int ch = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
-    const int n = a.n, p = a.p, sn = n + 1, sp = p + 1;
+    const int wv = tid >> 6, r = tid & 15, qd = (tid & 63) >> 4;
+    const int n = a.n, p = a.p, n4 = (n + 3) & ~3, sn = n4 + 1, sp = p + 1;
     float* qs = lds;
     float* Ss = qs + kCh * sn;
     const int start = a.ch_start[ch], len = a.ch_len[ch];
-    for (int i = tid; i < kCh * n; i += 256) {
-        const int t = i / n, j = i % n;
-        qs[t * sn + j] = t < len ? a.q[(int64_t)(start + t) * a.ldq + (int64_t)(h / a.q_div) * n + j] : 0.f;
+    for (int i = tid; i < kCh * n4; i += 256) {
+        const int t = i / n4, j = i % n4;
+        qs[t * sn + j] = (t < len && j < n) ? a.q[(int64_t)(start + t) * a.ldq + (int64_t)(h / a.q_div) * n + j] : 0.f;
     }
     const float* dsp = a.ds + ((int64_t)ch * a.H + h) * n * p;
-    for (int i = tid; i < n * p; i += 256) Ss[(i / p) * sp + i % p] = dsp[i];
+    for (int i = tid; i < n4 * p; i += 256) Ss[(i / p) * sp + i % p] = i < n * p ? dsp[i] : 0.f;
     __syncthreads();
-    const int tt = tid >> 4, cc = tid & 15;
+    // o[t][c] += exp(L_t) sum_j q[t][j] S0[j][c]: A = S0^T (columns c), B = q rows of the wave's tokens
+    const int t = 16 * wv + r;
     const float sk = a.skip ? a.skip[h] : 0.f;
-    for (int c0 = 0; c0 < p; c0 += 128) {
-        float acc[4][8] = {};
-        for (int j = 0; j < n; ++j) {
-            float qv[4], sv[8];
+    const float w = t < len ? expf(a.lsum[(int64_t)(start + t) * a.H + h]) : 0.f;
+    for (int c0 = 0; c0 < p; c0 += 64) {
+        f32x4_t o[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) qv[i] = qs[(tt * 4 + i) * sn + j];
+        for (int ct = 0; ct < 4; ++ct) o[ct] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        for (int j0 = 0; j0 < n4; j0 += 4) {
+            const float bq = qs[t * sn + j0 + qd];
+            const float* srow = Ss + (j0 + qd) * sp;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int c = c0 + cc + 16 * e;
-                sv[e] = c < p ? Ss[j * sp + c] : 0.f;
+            for (int ct = 0; ct < 4; ++ct) {
+                const int c = c0 + 16 * ct + r;
+                MV_MFMA4(o[ct], c < p ? srow[c] : 0.f, bq);
             }
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int e = 0; e < 8; ++e) acc[i][e] = fmaf(qv[i], sv[e], acc[i][e]);
         }
+        if (t < len) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int t = tt * 4 + i;
-            if (t >= len) continue;
-            const float w = expf(a.lsum[(int64_t)(start + t) * a.H + h]);
+            for (int ct = 0; ct < 4; ++ct)
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int c = c0 + cc + 16 * e;
-                if (c >= p) continue;
-                float* o = a.out + (int64_t)(start + t) * a.ldo + (int64_t)h * p + c;
-                float r = fmaf(w, acc[i][e], *o);
-                if (a.skip) r = fmaf(sk, a.v[(int64_t)(start + t) * a.ldv + (int64_t)h * p + c], r);
-                *o = r;
-            }
+                for (int j = 0; j < 4; ++j) {
+                    const int c = c0 + 16 * ct + 4 * qd + j;
+                    if (c >= p) continue;
+                    float* op = a.out + (int64_t)(start + t) * a.ldo + (int64_t)h * p + c;
+                    float res = fmaf(w, o[ct][j], *op);
+                    if (a.skip) res = fmaf(sk, a.v[(int64_t)(start + t) * a.ldv + (int64_t)h * p + c], res);
+                    *op = res;
+                }
         }
     }
 }
@@ -793,7 +781,10 @@ int mv_scan_outer(const float* q, int64_t ldq, int q_div, const float* k, int64_
 }
 
 size_t mv_scan_chunked_lds_bytes(int n, int p) {
-    return (size_t)(2 * mv::kCh * (n + 1) + mv::kCh * (p + 1) + mv::kCh * (mv::kCh + 1) + 2 * mv::kCh) * sizeof(float);
+    const int n4 = (n + 3) & ~3;
+    const size_t intra = (size_t)(2 * mv::kCh * (n4 + 1) + mv::kCh * (p + 1) + 2 * mv::kCh) * sizeof(float);
+    const size_t inter = (size_t)(mv::kCh * (n4 + 1) + n4 * (p + 1)) * sizeof(float);
+    return intra > inter ? intra : inter;
 }
 
 int mv_scan_chunked(const float* q, int64_t ldq, int q_div, const float* k, int64_t ldk, int k_div, const float* v,
@@ -808,9 +799,10 @@ int mv_scan_chunked(const float* q, int64_t ldq, int q_div, const float* k, int6
     if (!q || !k || !v || !log_decay || !state || !out || !ds || !lsum || !atot || !ch_start || !ch_len || !row_ch0 ||
         !row_nch || rows > 65535 || heads > 65535)
         return MV_ERR_INVALID_ARG;
-    const size_t lds = mv_scan_chunked_lds_bytes(n, p);
-    const size_t lds2 = (size_t)(kCh * (n + 1) + n * (p + 1)) * sizeof(float);
-    if (lds > 150 * 1024 || lds2 > 150 * 1024) return MV_ERR_UNSUPPORTED;
+    const int n4 = (n + 3) & ~3;
+    const size_t lds = (size_t)(2 * kCh * (n4 + 1) + kCh * (p + 1) + 2 * kCh) * sizeof(float);
+    const size_t lds2 = (size_t)(kCh * (n4 + 1) + n4 * (p + 1)) * sizeof(float);
+    if (mv_scan_chunked_lds_bytes(n, p) > 150 * 1024) return MV_ERR_UNSUPPORTED;
     static LdsOptIn opt1, opt2;
     if (int rc = ensure_dynamic_lds((const void*)scan_chunk_intra_kernel, lds, opt1)) return rc;
     if (int rc = ensure_dynamic_lds((const void*)scan_chunk_inter_kernel, lds2, opt2)) return rc;

@@ -165,7 +165,7 @@ def scan_outer(q, k, v, decay, gain, skip, state, out, step, heads: int, n: int,
     assert skip is None or (skip.numel() == heads and skip.is_contiguous())
     L = nv.lib()
     use_chunks = (chunked and log_decay is not None and step.n_chunks > 0
-                  and L.mv_scan_chunked_lds_bytes(n, p) <= 150 * 1024 and (64 * (n + 1) + n * (p + 1)) * 4 <= 150 * 1024)
+                  and L.mv_scan_chunked_lds_bytes(n, p) <= 150 * 1024)
     if use_chunks:
         assert log_decay.shape == decay.shape and log_decay.stride(-1) == 1
         dev = v.device
