@@ -522,15 +522,32 @@ __global__ __launch_bounds__(64 * NW) void window_attn_kernel(const float* q, in
         const int cnt = pos - j0 + 1 < 64 ? pos - j0 + 1 : 64;
 #pragma unroll
         for (int ci = 0; ci < kMaxVC; ++ci) acc[ci] *= corr;
-        for (int jj = 0; jj < cnt; ++jj) {
-            const int jk = j0 + jj;
-            const int pg = bt[jk / pr.page];
-            const T_* vr = vc + (((int64_t)pg * pr.page + jk % pr.page) * G + g) * dv;
-            const float pj = ps[jj];
+        // eight value rows at a time, their loads in flight together (a tile of 64 keys lies in two pages at
+        // most when a page holds 64 tokens or more: their ids are looked up once)
+        const int pA = j0 / pr.page;
+        const bool two = pr.page >= 64;
+        const int pgA = bt[pA], pgB = (two && (j0 + cnt - 1) / pr.page != pA) ? bt[pA + 1] : pgA;
+        for (int jj = 0; jj < cnt; jj += 8) {
+            float pj[8];
+            const T_* vr[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const bool ok = jj + u < cnt;
+                const int jk = ok ? j0 + jj + u : j0;
+                const int pg = two ? (jk / pr.page == pA ? pgA : pgB) : bt[jk / pr.page];
+                vr[u] = vc + (((int64_t)pg * pr.page + jk % pr.page) * G + g) * dv;
+                pj[u] = ok ? ps[jj + u] : 0.f;
+            }
 #pragma unroll
             for (int ci = 0; ci < kMaxVC; ++ci) {
                 const int c = lane + ci * 64;
-                if (c < dv) acc[ci] = fmaf(pj, ActS<F32>::ld(vr + c), acc[ci]);
+                if (c < dv) {
+                    float x[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) x[u] = ActS<F32>::ld(vr[u] + c);
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) acc[ci] = fmaf(pj[u], x[u], acc[ci]);
+                }
             }
         }
     }
