@@ -33,7 +33,7 @@ def step_of(cache, rows):
 
 
 @pytest.mark.parametrize("f32", [False, True])
-@pytest.mark.parametrize("m,n,k", [(1, 678, 256), (5, 37, 19), (70, 130, 288), (129, 64, 64), (3, 16, 2048)])
+@pytest.mark.parametrize("m,n,k", [(1, 650, 200), (5, 37, 19), (70, 130, 288), (129, 64, 64), (3, 16, 2048)])
 def test_linear_any(ops, f32, m, n, k):
     g = torch.Generator().manual_seed(m * 1000 + n)
     dt = torch.float32 if f32 else torch.bfloat16
