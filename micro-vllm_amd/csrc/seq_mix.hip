@@ -175,6 +175,7 @@ struct ChunkArgs {
     const int *ch_start, *ch_len, *row_ch0, *row_nch;
     StepRows r;
     int H, n, p;
+    int hb;   // heads of one group a workgroup takes in turn (they share q, k and the products q . k)
 };
 
 // All three products of a chunk run on v_mfma_f32_16x16x4_f32 (true fp32): operand A lane (r, g) = A[r][g],
@@ -183,7 +184,7 @@ struct ChunkArgs {
 
 __global__ __launch_bounds__(256) void scan_chunk_intra_kernel(ChunkArgs a) {
     extern __shared__ float lds[];
-    const int ch = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int ch = blockIdx.x, tid = threadIdx.x;
     const int wv = tid >> 6, r = tid & 15, qd = (tid & 63) >> 4;
     const int n = a.n, p = a.p, n4 = (n + 3) & ~3, sn = n4 + 1, sp = p + 1;
     float* qs = lds;
@@ -191,115 +192,119 @@ __global__ __launch_bounds__(256) void scan_chunk_intra_kernel(ChunkArgs a) {
     float* vs = ks + kCh * sn;
     float* Ls = vs + kCh * sp;
     float* gs = Ls + kCh;
+    float* ws = gs + kCh;
     const int start = a.ch_start[ch], len = a.ch_len[ch];
+    // a.hb heads of one group per workgroup: they share q and k, staged once, and the products q_t . k_s
+    const int h_first = blockIdx.y * a.hb;
     for (int i = tid; i < kCh * n4; i += 256) {
         const int t = i / n4, j = i % n4;
         const bool ok = t < len && j < n;
-        qs[t * sn + j] = ok ? a.q[(int64_t)(start + t) * a.ldq + (int64_t)(h / a.q_div) * n + j] : 0.f;
-        ks[t * sn + j] = ok ? a.k[(int64_t)(start + t) * a.ldk + (int64_t)(h / a.k_div) * n + j] : 0.f;
-    }
-    for (int i = tid; i < kCh * p; i += 256) {
-        const int t = i / p, c = i % p;
-        vs[t * sp + c] = t < len ? a.v[(int64_t)(start + t) * a.ldv + (int64_t)h * p + c] : 0.f;
-    }
-    if (tid < kCh) {   // one wave: inclusive running sum of the log decays
-        float l = 0.f, g = 0.f;
-        if (tid < len) {
-            l = fmaxf(a.log_decay[(int64_t)(start + tid) * a.ld_ld + h], -80.f);
-            g = a.gain ? a.gain[(int64_t)(start + tid) * a.ld_gain + h] : 1.f;
-        }
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-            const float up = __shfl_up(l, o, 64);
-            if (tid >= o) l += up;
-        }
-        Ls[tid] = l;
-        gs[tid] = g;
-        if (tid < len) a.lsum[(int64_t)(start + tid) * a.H + h] = l;
+        qs[t * sn + j] = ok ? a.q[(int64_t)(start + t) * a.ldq + (int64_t)(h_first / a.q_div) * n + j] : 0.f;
+        ks[t * sn + j] = ok ? a.k[(int64_t)(start + t) * a.ldk + (int64_t)(h_first / a.k_div) * n + j] : 0.f;
     }
     __syncthreads();
-    const float Lend = Ls[len - 1];
-    if (tid == 0) a.atot[(int64_t)ch * a.H + h] = expf(Lend);
-    // wave wv owns the tokens t = 16 wv + r.  P[nt][j] = P[t][s = 16 nt + 4 qd + j], s-tiles above the diagonal
-    // stay zero: A = k rows of the s-tile, B = q rows of the wave's tokens, summed over the state index
+    // wave wv owns the tokens t = 16 wv + r.  P0[nt][j] = q_t . k_s, s = 16 nt + 4 qd + j, s-tiles above the
+    // diagonal stay zero: A = k rows of the s-tile, B = q rows of the wave's tokens, summed over the state index
     const int t0 = 16 * wv, t = t0 + r;
-    f32x4_t P[4];
+    f32x4_t P0[4];
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt) P[nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int nt = 0; nt < 4; ++nt) P0[nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     for (int j0 = 0; j0 < n4; j0 += 4) {
         const float bq = qs[t * sn + j0 + qd];
 #pragma unroll
         for (int nt = 0; nt < 4; ++nt)
-            if (nt <= wv) MV_MFMA4(P[nt], ks[(16 * nt + r) * sn + j0 + qd], bq);
+            if (nt <= wv) MV_MFMA4(P0[nt], ks[(16 * nt + r) * sn + j0 + qd], bq);
     }
-    {
-        const float Lt = Ls[t];
-#pragma unroll
-        for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int s_ = 16 * nt + 4 * qd + j;
-                P[nt][j] = (s_ <= t) ? P[nt][j] * expf(Lt - Ls[s_]) * gs[s_] : 0.f;
-            }
-    }
-    // o[t][c] = sum_s P[t][s] v[s][c]: A = v^T (columns c), B = P straight from the registers
-    for (int c0 = 0; c0 < p; c0 += 64) {
-        f32x4_t o[4];
-#pragma unroll
-        for (int ct = 0; ct < 4; ++ct) o[ct] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int nt = 0; nt < 4; ++nt) {
-            if (nt > wv) continue;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float* vrow = vs + (16 * nt + 4 * qd + j) * sp;
-#pragma unroll
-                for (int ct = 0; ct < 4; ++ct) {
-                    const int c = c0 + 16 * ct + r;
-                    MV_MFMA4(o[ct], c < p ? vrow[c] : 0.f, P[nt][j]);
-                }
-            }
+    for (int hh = 0; hh < a.hb; ++hh) {
+        const int h = h_first + hh;
+        __syncthreads();   // the head before is done with vs, Ls, gs, ws
+        for (int i = tid; i < kCh * p; i += 256) {
+            const int tt = i / p, c = i % p;
+            vs[tt * sp + c] = tt < len ? a.v[(int64_t)(start + tt) * a.ldv + (int64_t)h * p + c] : 0.f;
         }
-        if (t < len) {
+        if (tid < kCh) {   // one wave: inclusive running sum of the log decays
+            float l = 0.f, g = 0.f;
+            if (tid < len) {
+                l = fmaxf(a.log_decay[(int64_t)(start + tid) * a.ld_ld + h], -80.f);
+                g = a.gain ? a.gain[(int64_t)(start + tid) * a.ld_gain + h] : 1.f;
+            }
 #pragma unroll
-            for (int ct = 0; ct < 4; ++ct)
+            for (int o = 1; o < 64; o <<= 1) {
+                const float up = __shfl_up(l, o, 64);
+                if (tid >= o) l += up;
+            }
+            Ls[tid] = l;
+            gs[tid] = g;
+            if (tid < len) a.lsum[(int64_t)(start + tid) * a.H + h] = l;
+            const float lend = __shfl(l, len - 1, 64);
+            ws[tid] = expf(lend - l) * g;        // weight of token s in the state the chunk ends with
+            if (tid == 0) a.atot[(int64_t)ch * a.H + h] = expf(lend);
+        }
+        __syncthreads();
+        f32x4_t P[4];
+        {
+            const float Lt = Ls[t];
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const int c = c0 + 16 * ct + 4 * qd + j;
-                    if (c < p) a.out[(int64_t)(start + t) * a.ldo + (int64_t)h * p + c] = o[ct][j];
+                    const int s_ = 16 * nt + 4 * qd + j;
+                    P[nt][j] = (s_ <= t) ? P0[nt][j] * expf(Lt - Ls[s_]) * gs[s_] : 0.f;
                 }
         }
-    }
-    // k_s <- k_s exp(L_end - L_s) gain_s, then dS[j][c] = sum_s k[s][j] v[s][c]: A = k^T, B = v, over the tokens
-    __syncthreads();
-    for (int i = tid; i < kCh * n4; i += 256) {
-        const int tt = i / n4, j = i % n4;
-        ks[tt * sn + j] *= expf(Lend - Ls[tt]) * gs[tt];
-    }
-    __syncthreads();
-    float* dsp = a.ds + ((int64_t)ch * a.H + h) * n * p;
-    for (int jt = wv; jt * 16 < n; jt += 4) {
-        const int ja = 16 * jt + r;
+        // o[t][c] = sum_s P[t][s] v[s][c]: A = v^T (columns c), B = P straight from the registers
         for (int c0 = 0; c0 < p; c0 += 64) {
-            f32x4_t dd[4];
+            f32x4_t o[4];
 #pragma unroll
-            for (int ct = 0; ct < 4; ++ct) dd[ct] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-            for (int s0 = 0; s0 < kCh; s0 += 4) {
-                const float ak = ja < n4 ? ks[(s0 + qd) * sn + ja] : 0.f;
-                const float* vrow = vs + (s0 + qd) * sp;
+            for (int ct = 0; ct < 4; ++ct) o[ct] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int ct = 0; ct < 4; ++ct) {
-                    const int c = c0 + 16 * ct + r;
-                    MV_MFMA4(dd[ct], ak, c < p ? vrow[c] : 0.f);
-                }
-            }
-#pragma unroll
-            for (int ct = 0; ct < 4; ++ct)
+            for (int nt = 0; nt < 4; ++nt) {
+                if (nt > wv) continue;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const int jj = 16 * jt + 4 * qd + j, c = c0 + 16 * ct + r;
-                    if (jj < n && c < p) dsp[(int64_t)jj * p + c] = dd[ct][j];
+                    const float* vrow = vs + (16 * nt + 4 * qd + j) * sp;
+#pragma unroll
+                    for (int ct = 0; ct < 4; ++ct) {
+                        const int c = c0 + 16 * ct + r;
+                        MV_MFMA4(o[ct], c < p ? vrow[c] : 0.f, P[nt][j]);
+                    }
                 }
+            }
+            if (t < len) {
+#pragma unroll
+                for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const int c = c0 + 16 * ct + 4 * qd + j;
+                        if (c < p) a.out[(int64_t)(start + t) * a.ldo + (int64_t)h * p + c] = o[ct][j];
+                    }
+            }
+        }
+        // dS[j][c] = sum_s (k[s][j] ws[s]) v[s][c]: A = k^T weighted as it is read, B = v, over the tokens
+        float* dsp = a.ds + ((int64_t)ch * a.H + h) * n * p;
+        for (int jt = wv; jt * 16 < n; jt += 4) {
+            const int ja = 16 * jt + r;
+            for (int c0 = 0; c0 < p; c0 += 64) {
+                f32x4_t dd[4];
+#pragma unroll
+                for (int ct = 0; ct < 4; ++ct) dd[ct] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+                for (int s0 = 0; s0 < kCh; s0 += 4) {
+                    const float ak = ja < n4 ? ks[(s0 + qd) * sn + ja] * ws[s0 + qd] : 0.f;
+                    const float* vrow = vs + (s0 + qd) * sp;
+#pragma unroll
+                    for (int ct = 0; ct < 4; ++ct) {
+                        const int c = c0 + 16 * ct + r;
+                        MV_MFMA4(dd[ct], ak, c < p ? vrow[c] : 0.f);
+                    }
+                }
+#pragma unroll
+                for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const int jj = 16 * jt + 4 * qd + j, c = c0 + 16 * ct + r;
+                        if (jj < n && c < p) dsp[(int64_t)jj * p + c] = dd[ct][j];
+                    }
+            }
         }
     }
 }
@@ -323,48 +328,54 @@ __global__ __launch_bounds__(256) void scan_chunk_carry_kernel(ChunkArgs a) {
 
 __global__ __launch_bounds__(256) void scan_chunk_inter_kernel(ChunkArgs a) {
     extern __shared__ float lds[];
-    const int ch = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int ch = blockIdx.x, tid = threadIdx.x;
     const int wv = tid >> 6, r = tid & 15, qd = (tid & 63) >> 4;
     const int n = a.n, p = a.p, n4 = (n + 3) & ~3, sn = n4 + 1, sp = p + 1;
     float* qs = lds;
     float* Ss = qs + kCh * sn;
     const int start = a.ch_start[ch], len = a.ch_len[ch];
+    const int h_first = blockIdx.y * a.hb;
     for (int i = tid; i < kCh * n4; i += 256) {
         const int t = i / n4, j = i % n4;
-        qs[t * sn + j] = (t < len && j < n) ? a.q[(int64_t)(start + t) * a.ldq + (int64_t)(h / a.q_div) * n + j] : 0.f;
+        qs[t * sn + j] =
+            (t < len && j < n) ? a.q[(int64_t)(start + t) * a.ldq + (int64_t)(h_first / a.q_div) * n + j] : 0.f;
     }
-    const float* dsp = a.ds + ((int64_t)ch * a.H + h) * n * p;
-    for (int i = tid; i < n4 * p; i += 256) Ss[(i / p) * sp + i % p] = i < n * p ? dsp[i] : 0.f;
-    __syncthreads();
-    // o[t][c] += exp(L_t) sum_j q[t][j] S0[j][c]: A = S0^T (columns c), B = q rows of the wave's tokens
     const int t = 16 * wv + r;
-    const float sk = a.skip ? a.skip[h] : 0.f;
-    const float w = t < len ? expf(a.lsum[(int64_t)(start + t) * a.H + h]) : 0.f;
-    for (int c0 = 0; c0 < p; c0 += 64) {
-        f32x4_t o[4];
+    for (int hh = 0; hh < a.hb; ++hh) {
+        const int h = h_first + hh;
+        __syncthreads();
+        const float* dsp = a.ds + ((int64_t)ch * a.H + h) * n * p;
+        for (int i = tid; i < n4 * p; i += 256) Ss[(i / p) * sp + i % p] = i < n * p ? dsp[i] : 0.f;
+        __syncthreads();
+        // o[t][c] += exp(L_t) sum_j q[t][j] S0[j][c]: A = S0^T (columns c), B = q rows of the wave's tokens
+        const float sk = a.skip ? a.skip[h] : 0.f;
+        const float w = t < len ? expf(a.lsum[(int64_t)(start + t) * a.H + h]) : 0.f;
+        for (int c0 = 0; c0 < p; c0 += 64) {
+            f32x4_t o[4];
 #pragma unroll
-        for (int ct = 0; ct < 4; ++ct) o[ct] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-        for (int j0 = 0; j0 < n4; j0 += 4) {
-            const float bq = qs[t * sn + j0 + qd];
-            const float* srow = Ss + (j0 + qd) * sp;
+            for (int ct = 0; ct < 4; ++ct) o[ct] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            for (int j0 = 0; j0 < n4; j0 += 4) {
+                const float bq = qs[t * sn + j0 + qd];
+                const float* srow = Ss + (j0 + qd) * sp;
 #pragma unroll
-            for (int ct = 0; ct < 4; ++ct) {
-                const int c = c0 + 16 * ct + r;
-                MV_MFMA4(o[ct], c < p ? srow[c] : 0.f, bq);
-            }
-        }
-        if (t < len) {
-#pragma unroll
-            for (int ct = 0; ct < 4; ++ct)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int c = c0 + 16 * ct + 4 * qd + j;
-                    if (c >= p) continue;
-                    float* op = a.out + (int64_t)(start + t) * a.ldo + (int64_t)h * p + c;
-                    float res = fmaf(w, o[ct][j], *op);
-                    if (a.skip) res = fmaf(sk, a.v[(int64_t)(start + t) * a.ldv + (int64_t)h * p + c], res);
-                    *op = res;
+                for (int ct = 0; ct < 4; ++ct) {
+                    const int c = c0 + 16 * ct + r;
+                    MV_MFMA4(o[ct], c < p ? srow[c] : 0.f, bq);
                 }
+            }
+            if (t < len) {
+#pragma unroll
+                for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const int c = c0 + 16 * ct + 4 * qd + j;
+                        if (c >= p) continue;
+                        float* op = a.out + (int64_t)(start + t) * a.ldo + (int64_t)h * p + c;
+                        float res = fmaf(w, o[ct][j], *op);
+                        if (a.skip) res = fmaf(sk, a.v[(int64_t)(start + t) * a.ldv + (int64_t)h * p + c], res);
+                        *op = res;
+                    }
+            }
         }
     }
 }
@@ -799,7 +810,7 @@ int mv_scan_outer(const float* q, int64_t ldq, int q_div, const float* k, int64_
 
 size_t mv_scan_chunked_lds_bytes(int n, int p) {
     const int n4 = (n + 3) & ~3;
-    const size_t intra = (size_t)(2 * mv::kCh * (n4 + 1) + mv::kCh * (p + 1) + 2 * mv::kCh) * sizeof(float);
+    const size_t intra = (size_t)(2 * mv::kCh * (n4 + 1) + mv::kCh * (p + 1) + 3 * mv::kCh) * sizeof(float);
     const size_t inter = (size_t)(mv::kCh * (n4 + 1) + n4 * (p + 1)) * sizeof(float);
     return intra > inter ? intra : inter;
 }
@@ -817,7 +828,7 @@ int mv_scan_chunked(const float* q, int64_t ldq, int q_div, const float* k, int6
         !row_nch || rows > 65535 || heads > 65535)
         return MV_ERR_INVALID_ARG;
     const int n4 = (n + 3) & ~3;
-    const size_t lds = (size_t)(2 * kCh * (n4 + 1) + kCh * (p + 1) + 2 * kCh) * sizeof(float);
+    const size_t lds = (size_t)(2 * kCh * (n4 + 1) + kCh * (p + 1) + 3 * kCh) * sizeof(float);
     const size_t lds2 = (size_t)(kCh * (n4 + 1) + n4 * (p + 1)) * sizeof(float);
     if (mv_scan_chunked_lds_bytes(n, p) > 150 * 1024) return MV_ERR_UNSUPPORTED;
     static LdsOptIn opt1, opt2;
@@ -830,10 +841,12 @@ int mv_scan_chunked(const float* q, int64_t ldq, int q_div, const float* k, int6
     a.ch_start = ch_start; a.ch_len = ch_len; a.row_ch0 = row_ch0; a.row_nch = row_nch;
     a.r = StepRows{nullptr, nullptr, nullptr, nullptr, row_ctx, row_slot};
     a.H = heads; a.n = n; a.p = p;
+    // heads that read the same q and k (a group) go four or two to a workgroup
+    a.hb = (q_div == k_div && heads % q_div == 0) ? (q_div % 4 == 0 ? 4 : (q_div % 2 == 0 ? 2 : 1)) : 1;
     hipStream_t s = (hipStream_t)stream;
-    hipLaunchKernelGGL(scan_chunk_intra_kernel, dim3(chunks, heads), dim3(256), lds, s, a);
+    hipLaunchKernelGGL(scan_chunk_intra_kernel, dim3(chunks, heads / a.hb), dim3(256), lds, s, a);
     hipLaunchKernelGGL(scan_chunk_carry_kernel, dim3((n * p + 255) / 256, heads, rows), dim3(256), 0, s, a);
-    hipLaunchKernelGGL(scan_chunk_inter_kernel, dim3(chunks, heads), dim3(256), lds2, s, a);
+    hipLaunchKernelGGL(scan_chunk_inter_kernel, dim3(chunks, heads / a.hb), dim3(256), lds2, s, a);
     return check_launch();
 }
 
