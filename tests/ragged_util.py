@@ -48,6 +48,41 @@ def config_b():
     ])
 
 
+def random_config(seed):
+    """A configuration drawn at random: layer order, borrowed weights, head counts and widths (among them the
+    shapes the matrix-core attention takes and ones it does not), windows from 1 to beyond the prompt, taps
+    from 1 to 5, groups, norm groups, rotation over none / part / all of a head, with and without soft cap."""
+    import random
+    rng = random.Random(seed)
+    layers = []
+    for i in range(rng.randint(2, 5)):
+        own = [k for k in range(i) if "weights_of" not in layers[k]]
+        if own and rng.random() < 0.3:
+            j = rng.choice(own)
+            layers.append(dict(layers[j], weights_of=j))
+            continue
+        ff = rng.choice([None, 64, 150, 256])
+        if rng.random() < 0.5:
+            groups = rng.choice([1, 2, 3])
+            heads = groups * rng.choice([1, 2, 4])
+            vdim = rng.choice([8, 20, 32, 48, 64])
+            ng = rng.choice([g for g in (1, 2, heads, groups) if (heads * vdim) % g == 0])
+            layers.append(layer("mamba2", mamba(heads, vdim, rng.choice([4, 6, 16, 48, 128]), groups, rng.randint(1, 5), ng), ff))
+        else:
+            kv = rng.choice([1, 2, 3])
+            dim, vdim = rng.choice([(8, 8), (24, 40), (32, 32), (64, 64), (96, 96), (128, 64), (64, 128), (40, 56), (128, 128)])
+            rh, rdim = rng.randint(1, 3), rng.choice([8, 16, 48, 64])
+            layers.append(layer("parallel", parallel(
+                heads=kv * rng.choice([1, 2, 4]), kv_heads=kv, dim=dim, vdim=vdim, window=rng.choice([1, 2, 17, 64, 65, 100, 300]),
+                scale=rng.choice([0.1, dim ** -0.5, 0.5]), r_heads=rh, r_dim=rdim, r_vdim=rng.choice([8, 20, 32, 64]),
+                rot=rng.choice([r for r in (0, 2, 8, 16, rdim) if r <= rdim]), base=rng.choice([100.0, 1e4, 1e6]),
+                decay=[rng.choice([0.5, 0.9, 0.99, 0.9995]) for _ in range(rh)], left_scale=rng.choice([0.5, 1.0, 1.7]),
+                right_scale=rng.choice([0.3, 1.0, 2.0])), ff))
+    return PagazenConfig(vocab_size=rng.choice([97, 256, 331, 1000]), width=rng.choice([48, 100, 192, 256]), layers=layers,
+                         embed_scale=rng.choice([1.0, 4.0, 16.0]), eps=rng.choice([1e-5, 1e-6]),
+                         logit_softcap=rng.choice([None, 15.0, 30.0]))
+
+
 def make_engine(cfg, dtype=torch.float32, seed=0, pages=24, slots=4, rows=4, step_tokens=512, max_tokens=512):
     from micro_vllm_amd.core.engine import InferenceEngine
     return InferenceEngine(model=build_random_model(cfg, seed), max_batch_size=rows, max_prefill_tokens=step_tokens,

@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from oracle import ref_hybrid as ref
-from ragged_util import config_a, config_b, make_engine, rel_err, run_in_portions
+from ragged_util import config_a, config_b, make_engine, random_config, rel_err, run_in_portions
 
 pytestmark = pytest.mark.gpu
 
@@ -73,6 +73,25 @@ def test_token_by_token_forms_agree_with_the_fast_ones():
                                   graphs=False)
         slow = run_in_portions(eng, "s", toks, [130, 50] + [1] * 20)
         assert rel_err(fast, slow) < tol
+
+
+@pytest.mark.parametrize("seed", [0, 4, 6, 9, 13, 16, 21, 33])
+def test_configurations_drawn_at_random(seed):
+    """Whole, in portions with a decoded tail, and two requests side by side, in fp32 against the
+    restatement; bf16 whole against decoding (the two must agree far better than either agrees with fp64:
+    some draws are ill-conditioned, their bf16 error is that of rounding the projections' inputs)."""
+    cfg = random_config(seed)
+    toks, other = tokens_for(cfg, 170, seed), tokens_for(cfg, 90, seed + 1000)
+    eng = make_engine(cfg, torch.float32, seed=seed, pages=16)
+    want, want2 = oracle_logits(eng, cfg, toks), oracle_logits(eng, cfg, other)
+    assert rel_err(run_in_portions(eng, "a", toks, [170]), want) < 1e-4
+    assert rel_err(run_in_portions(eng, "b", toks, [3, 64, 2, 40, 17] + [1] * 44), want) < 1e-4
+    o1 = eng.run_ragged([("c", toks[:100], list(range(100))), ("d", other[:20], list(range(20)))]).double().cpu()
+    o2 = eng.run_ragged([("c", toks[100:], list(range(70))), ("d", other[20:], list(range(70)))]).double().cpu()
+    assert rel_err(torch.cat([o1[:100], o2[:70]]), want) < 1e-4 and rel_err(torch.cat([o1[100:], o2[70:]]), want2) < 1e-4
+    eng = make_engine(cfg, torch.bfloat16, seed=seed, pages=16)
+    whole, tail = run_in_portions(eng, "a", toks, [170]), run_in_portions(eng, "b", toks, [100] + [1] * 70)
+    assert rel_err(whole, want) < 0.3 and rel_err(tail, whole) < 0.03
 
 
 def test_first_tokens_fp32():
