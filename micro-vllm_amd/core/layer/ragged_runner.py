@@ -194,10 +194,16 @@ class RaggedRunner:
     # ------------------------------------------------------------------ captured decoding steps
     def _replay(self, step: RaggedStep, cache: HybridCacheManager, want):
         B = step.rows
-        entry = self._graphs.get((B, id(cache)))
+        key = (B, id(cache))
+        if key not in self._graphs:
+            try:
+                self._graphs[key] = self._capture(step, cache)
+            except Exception as e:   # the recording failed (nothing of it ran): this row count stays uncaptured
+                logger.warning("decoding steps of %d rows are not captured: %r", B, e)
+                self._graphs[key] = None
+        entry = self._graphs[key]
         if entry is None:
-            entry = self._capture(step, cache)
-            self._graphs[(B, id(cache))] = entry
+            return self._run(step, cache, want, None)
         graph, logits = entry[0], entry[2]
         graph.replay()
         if want is None:
@@ -222,9 +228,11 @@ class RaggedRunner:
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             self._arena, self._measured = None, 0
-            self._run(step, cache, all_rows, None)
-            for t, old in saved:
-                t.index_copy_(0, idx, old)
+            try:
+                self._run(step, cache, all_rows, None)
+            finally:   # whatever that run did to the slots' state is undone: the step itself is still to come
+                for t, old in saved:
+                    t.index_copy_(0, idx, old)
             arena = torch.empty(self._measured + 4096, dtype=torch.uint8, device=self.device)
             side.synchronize()
             self._arena, self._arena_off = arena, 0

@@ -94,6 +94,23 @@ def test_configurations_drawn_at_random(seed):
     assert rel_err(whole, want) < 0.3 and rel_err(tail, whole) < 0.03
 
 
+def test_decoding_goes_on_when_a_step_cannot_be_captured(monkeypatch):
+    cfg = config_b()
+    eng = make_engine(cfg, torch.float32)
+    toks = tokens_for(cfg, 60, 17)
+    want = run_in_portions(eng, "w", toks, [60])
+    captured = run_in_portions(eng, "c", toks, [40] + [1] * 20)
+    assert any(v is not None for v in eng.runner._graphs.values())
+
+    def refuse(self, step, cache):
+        raise RuntimeError("no capture here")
+    monkeypatch.setattr(type(eng.runner), "_capture", refuse)
+    eng.runner._graphs.clear()
+    eager = run_in_portions(eng, "e", toks, [40] + [1] * 20)
+    assert list(eng.runner._graphs.values()) == [None]
+    assert rel_err(captured, want) < 2e-5 and rel_err(eager, want) < 2e-5
+
+
 def test_first_tokens_fp32():
     cfg = config_a()
     eng = make_engine(cfg, torch.float32)
