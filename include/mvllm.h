@@ -562,6 +562,90 @@ int mv_window_attn(const float* q, int64_t ldq, const void* k_cache, const void*
                    int window, int f32, const int32_t* row_len, const int32_t* ch_start, const int32_t* ch_len,
                    int chunks, int max_len, mv_stream_t stream);
 
+/* ---- further row-wise steps of fp32-stream stacks (stream_ops.hip) ---------------------------------- */
+
+/* n = tanh(alpha x) w + b (a norm that forms no statistics); h_t = act( n_t + (n_(t-1) - n_t) * mix ): every
+ * token's normed vector blended with its predecessor's.  The predecessor of a row's first token is the vector
+ * kept in state[slot] (zeros when row_ctx == 0); the row's last n is left there for its next step. */
+int mv_dyt_shift(const float* x, int64_t ldx, const float* w, const float* b, const float* alpha, const float* mix,
+                 float* state, void* h, int64_t ldh, const int32_t* tok_row, const int32_t* row_start,
+                 const int32_t* row_len, const int32_t* row_ctx, const int32_t* row_slot, int tokens, int n, int f32,
+                 mv_stream_t stream);
+/* out[r,:] = act( tanh(alpha x[idx[r],:]) w + b ); idx == NULL: row r itself. */
+int mv_dyt_gather(const float* x, int64_t ldx, const int32_t* idx, const float* w, const float* b, const float* alpha,
+                  void* out, int64_t ldo, int rows, int n, int f32, mv_stream_t stream);
+/* x += tanh(alpha y) w + b; h = act(x) unless h == NULL. */
+int mv_dyt_residual(const float* y, int64_t ldy, const float* w, const float* b, const float* alpha, float* x,
+                    int64_t ldx, void* h, int64_t ldh, int rows, int n, int f32, mv_stream_t stream);
+/* x += y / sqrt(mean(y^2) + eps) * w (plain weight); h = act(x) unless h == NULL. */
+int mv_unitnorm_residual(const float* y, int64_t ldy, const float* w, float eps, float* x, int64_t ldx, void* h,
+                         int64_t ldh, int rows, int n, int f32, mv_stream_t stream);
+/* `per` groups of n values in each of `rows` rows: out = act( v / sqrt(mean(v^2) + eps) * w ), w [n] shared. */
+int mv_rmsnorm_rows(const float* v, int64_t ld, int per, const float* w, float eps, void* out, int64_t ldo,
+                    int rows, int n, int f32, mv_stream_t stream);
+/* out[r,:] = act( gelu_tanh(a[r,:]) * table[ids[r]][off .. off+n) ), table rows of ldt values. */
+int mv_gelu_gate_rows(const float* a, int64_t lda, const void* table, int64_t ldt, int off, const int32_t* ids,
+                      int vocab, void* out, int64_t ldo, int rows, int n, int f32, mv_stream_t stream);
+/* out = act( silu(a[:, :n]) * a[:, n:2n] ). */
+int mv_silu_mul(const float* a, int64_t lda, void* out, int64_t ldo, int rows, int n, int f32, mv_stream_t stream);
+/* out = act( a * sigmoid(g) ); g == NULL: act(a). */
+int mv_sigmoid_gate(const float* a, int64_t lda, const float* g, int64_t ldg, void* out, int64_t ldo, int rows, int n,
+                    int f32, mv_stream_t stream);
+
+/* ---- products per head and per segment (linear_any.hip) --------------------------------------------- */
+
+/* `heads` products in one launch: y[:, h*zy .. +n] = x[:, h*zx .. +k] . W_h^T, W_h = w + h*zw ([n,k], row stride ldw). */
+int mv_linear_heads(const void* x, int64_t ldx, int64_t zx, const void* w, int64_t ldw, int64_t zw, float* y,
+                    int64_t ldy, int64_t zy, int m, int n, int k, int heads, int f32, mv_stream_t stream);
+/* Output rows seg[e] .. seg[e+1] use weight w + e*zw; operand row of output row i is src[i] / src_div (src == NULL:
+ * i).  max_rows bounds the rows of one segment. */
+int mv_linear_segments(const void* x, int64_t ldx, const void* w, int64_t ldw, int64_t zw, float* y, int64_t ldy,
+                       const int32_t* seg, const int32_t* src, int src_div, int segments, int max_rows, int n, int k,
+                       int f32, mv_stream_t stream);
+
+/* ---- gated recurrence without a key (seq_mix.hip) ---------------------------------------------------- */
+
+/* q = silu(q), f = lower + (1 - lower) * sigmoid(f + bias) in place ([tokens, n] each, bias may be NULL). */
+int mv_gate_lower_bound(float* q, int64_t ldq, float* f, int64_t ldf, const float* bias, const float* lower,
+                        int tokens, int n, mv_stream_t stream);
+/* S_t = diag(f_t) S_(t-1) + (1 - f_t) v_t^T, o_t = S_t^T q_t per head; q, f [T, heads*n], v, out [T, heads*p],
+ * state [slots, heads, n, p] fp32 (taken as zero when row_ctx == 0). */
+int mv_scan_gated(const float* q, int64_t ldq, const float* f, int64_t ldf, const float* v, int64_t ldv, float* state,
+                  float* out, int64_t ldo, const int32_t* row_start, const int32_t* row_len, const int32_t* row_ctx,
+                  const int32_t* row_slot, int rows, int heads, int n, int p, mv_stream_t stream);
+
+/* ---- attention over a cached latent (latent_attn.hip) ------------------------------------------------ */
+
+/* Per token: cache[page row] = [ unit-RMS(dkv[:rank]) * w_norm | rotate(dkv[rank : rank + r]) ] in the activation
+ * type; q_plain[t, h*d ..] = act(q[t, h*(d+r) .. +d]); q_abs[t, h*(rank+r) + rank ..] = rotate(q[t, h*(d+r) + d ..]).
+ * Rotation by the token's position over the first `rot` of the r dimensions, pairs (2i, 2i+1) when `interleaved`,
+ * else (i, i + rot/2); inv_freq [rot/2] fp64. */
+int mv_latent_prep(const float* dkv, int64_t ldkv, const float* w_norm, float eps, void* cache, const float* q,
+                   int64_t ldq, void* q_plain, int64_t ldqn, float* q_abs, int64_t ldqa, const double* inv_freq,
+                   const int32_t* tok_row, const int32_t* tok_pos, const int32_t* block_table, int bt_stride, int page,
+                   int tokens, int heads, int d, int r, int rank, int rot, int interleaved, int f32,
+                   mv_stream_t stream);
+/* out[t, h*rank ..] = sum_j softmax_j( q_abs[t,h] . cache[j] * scale ) cache[j][:rank] over the keys j <= position
+ * (window > 0: only the last `window` of them); sinks != NULL: exp(sinks[h]) joins the denominator. */
+int mv_latent_attn(const float* q_abs, int64_t ldq, const void* cache, void* out, int64_t ldo, const int32_t* tok_row,
+                   const int32_t* tok_pos, const int32_t* block_table, int bt_stride, int page, const float* sinks,
+                   int tokens, int heads, int rank, int r, float scale, int window, int f32, mv_stream_t stream);
+
+/* ---- routed experts (moe.hip) ------------------------------------------------------------------------ */
+
+/* ids / weights [tokens, top]: the `top` largest of W_router h (fp32; ties to the lower index) and the softmax over
+ * them; shared_gate[t] = sigmoid(w_shared_gate . h_t) when w_shared_gate != NULL. */
+int mv_moe_route(const void* h, int64_t ldh, const float* w_router, const float* w_shared_gate, int32_t* ids,
+                 float* weights, float* shared_gate, int tokens, int n, int experts, int top, int f32,
+                 mv_stream_t stream);
+/* (token, choice) pairs sorted by expert: seg [experts + 1], order [pairs] (pair in each row), place [pairs]. */
+int mv_moe_plan(const int32_t* ids, int32_t* seg, int32_t* order, int32_t* place, int pairs, int experts,
+                mv_stream_t stream);
+/* y_t = sum_k weights[t,k] * expert_out[place[t*top+k]] (+ shared_gate[t] * shared_out[t]). */
+int mv_moe_combine(const float* expert_out, int64_t lde, const int32_t* place, const float* weights,
+                   const float* shared_out, int64_t lds, const float* shared_gate, float* y, int64_t ldy, int tokens,
+                   int n, int top, mv_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

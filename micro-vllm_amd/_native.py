@@ -109,6 +109,24 @@ PROTOTYPES = {
     "mv_qk_unitnorm_store": (_I, [_P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P]),
     "mv_window_attn": (_I, [_P, _L, _P, _P, _P, _L, _P, _P, _P, _I, _I, _P, _I, _I, _I, _I, _I, _F, _I, _I,
                             _P, _P, _P, _I, _I, _P]),
+    "mv_dyt_shift": (_I, [_P, _L, _P, _P, _P, _P, _P, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _P]),
+    "mv_dyt_gather": (_I, [_P, _L, _P, _P, _P, _P, _P, _L, _I, _I, _I, _P]),
+    "mv_dyt_residual": (_I, [_P, _L, _P, _P, _P, _P, _L, _P, _L, _I, _I, _I, _P]),
+    "mv_unitnorm_residual": (_I, [_P, _L, _P, _F, _P, _L, _P, _L, _I, _I, _I, _P]),
+    "mv_rmsnorm_rows": (_I, [_P, _L, _I, _P, _F, _P, _L, _I, _I, _I, _P]),
+    "mv_gelu_gate_rows": (_I, [_P, _L, _P, _L, _I, _P, _I, _P, _L, _I, _I, _I, _P]),
+    "mv_silu_mul": (_I, [_P, _L, _P, _L, _I, _I, _I, _P]),
+    "mv_sigmoid_gate": (_I, [_P, _L, _P, _L, _P, _L, _I, _I, _I, _P]),
+    "mv_linear_heads": (_I, [_P, _L, _L, _P, _L, _L, _P, _L, _L, _I, _I, _I, _I, _I, _P]),
+    "mv_linear_segments": (_I, [_P, _L, _P, _L, _L, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
+    "mv_gate_lower_bound": (_I, [_P, _L, _P, _L, _P, _P, _I, _I, _P]),
+    "mv_scan_gated": (_I, [_P, _L, _P, _L, _P, _L, _P, _P, _L, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "mv_latent_prep": (_I, [_P, _L, _P, _F, _P, _P, _L, _P, _L, _P, _L, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I,
+                            _I, _I, _I, _P]),
+    "mv_latent_attn": (_I, [_P, _L, _P, _P, _L, _P, _P, _P, _I, _I, _P, _I, _I, _I, _I, _F, _I, _I, _P]),
+    "mv_moe_route": (_I, [_P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
+    "mv_moe_plan": (_I, [_P, _P, _P, _P, _I, _I, _P]),
+    "mv_moe_combine": (_I, [_P, _L, _P, _P, _P, _L, _P, _P, _L, _I, _I, _I, _P]),
     "mv_graph_begin_capture": (_I, [_P]),
     "mv_graph_end_capture": (_I, [_P, ctypes.POINTER(c_void_p)]),
     "mv_graph_launch": (_I, [_P, _P]),

@@ -29,6 +29,8 @@ SOURCES = [
     "linear_any.hip",
     "stream_ops.hip",
     "seq_mix.hip",
+    "latent_attn.hip",
+    "moe.hip",
 ]
 
 # Libraries that hold a part of the sources, `lib/libmvllm_<name>.so`: what one model family needs, for a
@@ -37,8 +39,8 @@ SOURCES = [
 SETS = {
     # fp32 residual stream, recurrent mixers, windowed attention; the wave-tile projections for the
     # shapes they take, and the sampler
-    "ragged": ["runtime.hip", "linear_any.hip", "stream_ops.hip", "seq_mix.hip", "elementwise.hip", "wgemm.hip",
-               "gemm_prefill.hip", "sampler.hip"],
+    "ragged": ["runtime.hip", "linear_any.hip", "stream_ops.hip", "seq_mix.hip", "latent_attn.hip", "moe.hip",
+               "elementwise.hip", "wgemm.hip", "gemm_prefill.hip", "sampler.hip"],
 }
 
 # -ffp-contract=off: rounding is part of the parity contract; FMAs are written explicitly
@@ -66,6 +68,8 @@ FILE_FLAGS = {
     "linear_any.hip": _NO_PACKED_F32,
     "stream_ops.hip": _NO_PACKED_F32,
     "seq_mix.hip": _NO_PACKED_F32,
+    "latent_attn.hip": _NO_PACKED_F32,
+    "moe.hip": _NO_PACKED_F32,
 }
 
 

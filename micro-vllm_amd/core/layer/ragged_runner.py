@@ -17,6 +17,23 @@ Per layer (Pagazen):
             unit-RMS per head, SiLU(g) gate -> out-projection
   then      x += unit_rms(sublayer output) * (1 + w)  (both mixers of a parallel layer enter one norm)
   mlp       up -> relu^2 -> down -> the same post-norm residual step
+
+Per layer (Fagunex; norms are Dynamic Tanh, before and after each sublayer):
+  every mixer reads  act( n + (n_prev - n) * shift ), n = norm1(x): norm and token shift in one launch, the
+            last n of a row kept per slot
+  hgrn2     fused q|f|v projection -> silu(q), f = lower + (1 - lower) sigmoid(f + b) -> gated scan with
+            key 1 - f (state per slot) -> unit-RMS per head, weight -> out-projection
+  latent attention (both kinds)  fused [dq|]dkv[|g] projection -> (kind 1: unit-RMS of the query latent ->
+            up-projection; kind 2: q in the fused projection) -> latent normed and rotated key part into the
+            page, q's rotated part rotated -> per-head product carrying q's unrotated part into the latent
+            space -> attention over the cached latents (window / causal, sink or none) -> per-head value
+            up-projection -> (sigmoid gate,) cast -> out-projection
+  then      x += norm1b(mixer output)
+  moe       norm2 -> router (fp32, top-k, softmax over the chosen, shared expert's sigmoid) -> (token, choice)
+            pairs sorted by expert -> gate|up by segment -> SiLU-gate -> down by segment; shared expert
+            gate|up -> SiLU-gate -> down; weighted sum -> x += norm2b(sum)
+  side      gate projection of x -> gelu_tanh * slice of the second embedding -> projection ->
+            x += unit-RMS * weight
 """
 import logging
 from typing import Dict, List, Optional
@@ -24,7 +41,7 @@ from typing import Dict, List, Optional
 import torch
 
 from ...kernel import ragged_ops as ops
-from ...models.pagazen import PagazenConfig, mamba2_sizes
+from ...models.pagazen import mamba2_sizes
 from ..state_cache import HybridCacheManager, RaggedStep
 
 logger = logging.getLogger(__name__)
@@ -47,15 +64,22 @@ class RaggedRunner:
         self._arena, self._arena_off, self._measured = None, 0, 0
         self.model, self.cfg, self.device, self.dtype = model, model.config, device, dtype
         self.wave_tiles = wave_tiles
-        cfg: PagazenConfig = self.cfg
+        cfg = self.cfg
         self.vocab_size, self.width = cfg.vocab_size, cfg.width
         self.weight_bytes = 0
         self._w: Dict[int, dict] = {}
-        for i, layer in enumerate(cfg.layers):
-            if cfg.weights_layer(i) == i:
-                self._w[i] = self._prepare_layer(i, layer)
+        # a layer RUN = (layer whose tensors it uses, its description); every run has a cache / state of its own
+        self.runs = cfg.layer_runs()
+        self.sandwich = cfg.architecture == "Fagunex"     # Dynamic Tanh before and after each sublayer
+        for wi, layer in self.runs:
+            if wi not in self._w:
+                self._w[wi] = self._prepare_layer(wi, layer)
         self.embed = self._act(model.get("embed"))
-        self.final_norm = self._small(model.get("final.norm"))
+        if self.sandwich:
+            self.final_norm = self._dyt_norm("final.norm")
+            self.side_embed = self._act(model.get("side.embed")) if cfg.side_dim else None
+        else:
+            self.final_norm = self._small(model.get("final.norm"))
         self.head = self._linear(model.get("head"))
 
     # ------------------------------------------------------------------ weights
@@ -71,7 +95,19 @@ class RaggedRunner:
         self.weight_bytes += lin.nbytes
         return lin
 
+    def _dyt_norm(self, name):
+        g = self.model.get
+        return (self._small(g(name)), self._small(g(name + ".b")), self._small(g(name + ".alpha")).reshape(1))
+
+    def _stacked(self, parts):
+        """[E, n, k] in the activation type: the same projection of several experts or heads."""
+        w = torch.stack([self._act(p) for p in parts], dim=0).contiguous()
+        self.weight_bytes += w.numel() * w.element_size()
+        return w
+
     def _prepare_layer(self, i: int, layer: dict) -> dict:
+        if self.sandwich:
+            return self._prepare_fagunex(i, layer)
         g, p, m = self.model.get, f"l{i}.", layer["mixer"]
         w = {"norm1": self._small(g(p + "norm1"))}
         if layer["type"] == "mamba2":
@@ -99,15 +135,60 @@ class RaggedRunner:
                      down=self._linear(g(p + "mlp.down")))
         return w
 
+    def _prepare_fagunex(self, i: int, layer: dict) -> dict:
+        g, p, m, cfg = self.model.get, f"l{i}.", layer["mixer"], self.cfg
+        w = {"norm1": self._dyt_norm(p + "norm1"), "norm1b": self._dyt_norm(p + "norm1b"),
+             "shift": self._small(g(p + "shift"))}
+        H = int(m["heads"])
+        if layer["type"] == "hgrn2":
+            w.update(qfv=self._linear(g(p + "mix.q"), g(p + "mix.f"), g(p + "mix.v")), f_b=self._small(g(p + "mix.f.b")),
+                     lower=self._small(g(p + "mix.lower")), norm=self._small(g(p + "mix.norm")),
+                     w_o=self._linear(g(p + "mix.o")))
+        else:
+            d, r, dv, R = int(m["dim"]), int(m["rot_dim"]), int(m["vdim"]), int(m["kv_rank"])
+            rot = int(m["rot"]["dims"]) if m.get("rot") else 0
+            base = float(m["rot"]["base"]) if rot else 1.0
+            inv_freq = base ** (-2.0 * torch.arange(max(rot // 2, 1), dtype=torch.float64) / max(rot, 1))
+            if layer["type"] == "latent_attention":
+                w.update(w_in=self._linear(g(p + "mix.dq"), g(p + "mix.dkv"), g(p + "mix.g")),
+                         q_norm=self._small(g(p + "mix.dq.norm")), w_uq=self._linear(g(p + "mix.uq")),
+                         sink=self._small(g(p + "mix.sink")))
+            else:
+                w.update(w_in=self._linear(g(p + "mix.q"), g(p + "mix.dkv")))
+            # per head: q_abs = W_uk,h^T q (so the stacked weight is [H, R, d]), value = W_uv,h * latent sum ([H, dv, R])
+            uk = g(p + "mix.uk").reshape(H, d, R).transpose(1, 2)
+            uv = g(p + "mix.uv").reshape(H, dv, R)
+            w.update(kv_norm=self._small(g(p + "mix.dkv.norm")), uk_t=self._stacked(list(uk)), uv=self._stacked(list(uv)),
+                     w_o=self._linear(g(p + "mix.o")), inv_freq=inv_freq.to(self.device), rot=rot)
+        mlp = layer.get("mlp")
+        if mlp:
+            E = int(mlp["router"]["experts"])
+            w.update(norm2=self._dyt_norm(p + "norm2"), norm2b=self._dyt_norm(p + "norm2b"),
+                     router=self._small(g(p + "mlp.router")),
+                     e_gu=self._stacked([torch.cat([g(p + f"mlp.e{e}.gate"), g(p + f"mlp.e{e}.up")], dim=0) for e in range(E)]),
+                     e_down=self._stacked([g(p + f"mlp.e{e}.down") for e in range(E)]))
+            if mlp.get("shared"):
+                w.update(s_gu=self._linear(g(p + "mlp.shared.gate"), g(p + "mlp.shared.up")),
+                         s_down=self._linear(g(p + "mlp.shared.down")), s_gate=self._small(g(p + "mlp.shared.sg")).reshape(-1))
+        if cfg.side_dim:
+            w.update(side_gate=self._linear(g(p + "side.gate")), side_proj=self._linear(g(p + "side.proj")),
+                     side_norm=self._small(g(p + "side.norm")), side_off=i * cfg.side_dim)
+        return w
+
     # ------------------------------------------------------------------ cache geometry
     def cache_layout(self):
         """(kv_layers, state_layers) for HybridCacheManager: what every layer RUN keeps per sequence."""
         kv, state = {}, {}
-        for i, layer in enumerate(self.cfg.layers):
+        for i, (_, layer) in enumerate(self.runs):
             m = layer["mixer"]
             if layer["type"] == "mamba2":
                 s = mamba2_sizes(m)
                 state[i] = {"conv": (max(s["taps"] - 1, 0), s["conv_ch"]), "ssm": (s["heads"], s["n"], s["p"])}
+            elif layer["type"] == "hgrn2":
+                state[i] = {"shift": (self.width,), "gated": (int(m["heads"]), int(m["dim"]), int(m["vdim"]))}
+            elif layer["type"] in ("latent_attention", "latent_attention_2"):
+                kv[i] = (1, int(m["kv_rank"]) + int(m["rot_dim"]), 0)    # one latent + rotated key part per token
+                state[i] = {"shift": (self.width,)}
             else:
                 L, R = m["left"], m["right"]
                 kv[i] = (int(L["kv_heads"]), int(L["dim"]), int(L["vdim"]))
@@ -251,29 +332,125 @@ class RaggedRunner:
     def _run(self, step: RaggedStep, cache: HybridCacheManager, want, residuals) -> torch.Tensor:
         cfg, T = self.cfg, step.tokens
         x, h = self._f32buf(T, self.width), self._actbuf(T, self.width)
-        ops.embed_scaled(self.embed, step.ids, cfg.embed_scale, x, h)
-        for li, layer in enumerate(cfg.layers):
-            w, m = self._w[cfg.weights_layer(li)], layer["mixer"]
-            if layer["type"] == "mamba2":
-                y1, y2 = self._mamba2(li, w, h, step, cache)
-                ops.postnorm_residual(y1, w["norm1"], cfg.eps, x, h)
-            else:
-                y1, y2 = self._parallel(li, w, m, h, step, cache)
-                ops.postnorm_residual(y1, w["norm1"], cfg.eps, x, h, y2=y2, s1=float(m["left_scale"]),
-                                      s2=float(m["right_scale"]))
-            if layer.get("mlp"):
-                up = w["up"](h, self._f32buf(T, w["up"].n))
-                act = self._actbuf(T, up.shape[1])
-                ops.relu_squared(up, act)
-                ops.postnorm_residual(w["down"](act, self._f32buf(T, self.width)), w["norm2"], cfg.eps, x, h)
-            if residuals is not None:
-                residuals.append(x.clone())
+        if self.sandwich:
+            ops.embed_scaled(self.embed, step.ids, 1.0, x, h)
+            for li, (wi, layer) in enumerate(self.runs):
+                self._fagunex_layer(li, self._w[wi], layer, x, h, step, cache)
+                if residuals is not None:
+                    residuals.append(x.clone())
+        else:
+            ops.embed_scaled(self.embed, step.ids, cfg.embed_scale, x, h)
+            for li, (wi, layer) in enumerate(self.runs):
+                w, m = self._w[wi], layer["mixer"]
+                if layer["type"] == "mamba2":
+                    y1, y2 = self._mamba2(li, w, h, step, cache)
+                    ops.postnorm_residual(y1, w["norm1"], cfg.eps, x, h)
+                else:
+                    y1, y2 = self._parallel(li, w, m, h, step, cache)
+                    ops.postnorm_residual(y1, w["norm1"], cfg.eps, x, h, y2=y2, s1=float(m["left_scale"]),
+                                          s2=float(m["right_scale"]))
+                if layer.get("mlp"):
+                    up = w["up"](h, self._f32buf(T, w["up"].n))
+                    act = self._actbuf(T, up.shape[1])
+                    ops.relu_squared(up, act)
+                    ops.postnorm_residual(w["down"](act, self._f32buf(T, self.width)), w["norm2"], cfg.eps, x, h)
+                if residuals is not None:
+                    residuals.append(x.clone())
         rows = T if want is None else want.numel()
         normed = self._actbuf(rows, self.width)
         if rows == 0:
             return self._f32buf(0, self.vocab_size)
-        ops.offset_rmsnorm_gather(x, want, self.final_norm, cfg.eps, normed)
+        if self.sandwich:
+            ops.dyt_gather(x, want, self.final_norm, normed)
+        else:
+            ops.offset_rmsnorm_gather(x, want, self.final_norm, cfg.eps, normed)
         logits = self.head(normed, self._f32buf(rows, self.vocab_size))
-        if cfg.logit_softcap:
+        if getattr(cfg, "logit_softcap", None):
             ops.softcap_(logits, cfg.logit_softcap)
         return logits
+
+    # ------------------------------------------------------------------ Fagunex layers
+    def _i32buf(self, count):
+        return self._take(1, count, torch.float32).view(torch.int32).view(-1)
+
+    def _fagunex_layer(self, li, w, layer, x, h, step: RaggedStep, cache: HybridCacheManager):
+        """One layer run on the stream x (fp32, updated in place); h is scratch of the activation type."""
+        T, cfg = step.tokens, self.cfg
+        ops.dyt_shift(x, w["norm1"], w["shift"], cache.states[li]["shift"], h, step)
+        if layer["type"] == "hgrn2":
+            y = self._hgrn2(li, w, layer["mixer"], h, step, cache)
+        else:
+            y = self._latent_attention(li, w, layer["mixer"], h, step, cache, layer["type"] == "latent_attention")
+        mlp = layer.get("mlp")
+        # the copy of x in the activation type is what the side input's gate reads when no feed-forward follows
+        ops.dyt_residual(y, w["norm1b"], x, h if (not mlp and cfg.side_dim) else None)
+        if mlp:
+            ops.dyt_gather(x, None, w["norm2"], h)
+            y = self._moe(w, mlp, h, T)
+            ops.dyt_residual(y, w["norm2b"], x, h if cfg.side_dim else None)
+        if cfg.side_dim:
+            a = w["side_gate"](h, self._f32buf(T, cfg.side_dim))
+            g = self._actbuf(T, cfg.side_dim)
+            ops.gelu_gate_rows(a, self.side_embed, w["side_off"], step.ids, g)
+            ops.unitnorm_residual(w["side_proj"](g, self._f32buf(T, self.width)), w["side_norm"], cfg.eps, x)
+
+    def _hgrn2(self, li, w, m, h, step: RaggedStep, cache: HybridCacheManager):
+        T, H, n, p = step.tokens, int(m["heads"]), int(m["dim"]), int(m["vdim"])
+        proj = w["qfv"](h, self._f32buf(T, w["qfv"].n))               # [q | f | v]
+        q, f, v = proj[:, :H * n], proj[:, H * n:2 * H * n], proj[:, 2 * H * n:]
+        ops.gate_lower_bound_(q, f, w["f_b"], w["lower"])
+        o = self._f32buf(T, H * p)
+        ops.scan_gated(q, f, v, cache.states[li]["gated"], o, step, H, n, p)
+        u = self._actbuf(T, H * p)
+        ops.rmsnorm_rows(o, w["norm"], self.cfg.eps, u, per=H)
+        return w["w_o"](u, self._f32buf(T, self.width))
+
+    def _latent_attention(self, li, w, m, h, step: RaggedStep, cache: HybridCacheManager, first_kind: bool):
+        T, eps = step.tokens, self.cfg.eps
+        H, d, r, dv, R = int(m["heads"]), int(m["dim"]), int(m["rot_dim"]), int(m["vdim"]), int(m["kv_rank"])
+        proj = w["w_in"](h, self._f32buf(T, w["w_in"].n))
+        if first_kind:        # [dq | dkv | g]: queries through a normed latent
+            Q = int(m["q_rank"])
+            cq = self._actbuf(T, Q)
+            ops.rmsnorm_rows(proj[:, :Q], w["q_norm"], eps, cq)
+            q = w["w_uq"](cq, self._f32buf(T, H * (d + r)))
+            dkv, gate = proj[:, Q:Q + R + r], proj[:, Q + R + r:]
+            window, sink = int(m["mask"]["size"]), w["sink"]
+        else:                 # [q | dkv]
+            q, dkv, gate = proj[:, :H * (d + r)], proj[:, H * (d + r):], None
+            window, sink = 0, None
+        pages = cache.k_caches[li]
+        pages = pages.view(pages.shape[0], pages.shape[1], R + r)
+        q_plain, q_abs = self._actbuf(T, H * d), self._f32buf(T, H * (R + r))
+        ops.latent_prep(dkv, w["kv_norm"], eps, pages, q, q_plain, q_abs, w["inv_freq"], step, H, d, r, R, w["rot"],
+                        interleaved=first_kind)
+        ops.linear_heads(q_plain, w["uk_t"], q_abs.view(T, H, R + r)[:, :, :R], H)
+        lat = self._actbuf(T, H * R)
+        ops.latent_attn(q_abs, pages, lat, step, sink, H, R, r, float(m["scale"]), window)
+        val = self._f32buf(T, H * dv)
+        ops.linear_heads(lat, w["uv"], val.view(T, H, dv), H)
+        a = self._actbuf(T, H * dv)
+        ops.sigmoid_gate(val, gate, a)
+        return w["w_o"](a, self._f32buf(T, self.width))
+
+    def _moe(self, w, mlp, h, T):
+        E, top, ff = int(mlp["router"]["experts"]), int(mlp["router"]["top"]), int(mlp["expert"]["ff"])
+        shared = mlp.get("shared")
+        ids = self._i32buf(T * top).view(T, top)
+        wts, sgate = self._f32buf(T, top), self._f32buf(1, T).view(-1)
+        ops.moe_route(h, w["router"], w["s_gate"] if shared else None, ids, wts, sgate)
+        seg, order, place = self._i32buf(E + 1), self._i32buf(T * top), self._i32buf(T * top)
+        ops.moe_plan(ids, seg, order, place, E)
+        gu = ops.linear_segments(h, w["e_gu"], self._f32buf(T * top, 2 * ff), seg, order, top, T)
+        act = self._actbuf(T * top, ff)
+        ops.silu_mul(gu, act)
+        down = ops.linear_segments(act, w["e_down"], self._f32buf(T * top, self.width), seg, None, 1, T)
+        s_out = None
+        if shared:
+            sf = int(shared["ff"])
+            s_act = self._actbuf(T, sf)
+            ops.silu_mul(w["s_gu"](h, self._f32buf(T, 2 * sf)), s_act)
+            s_out = w["s_down"](s_act, self._f32buf(T, self.width))
+        y = self._f32buf(T, self.width)
+        ops.moe_combine(down, place, wts, s_out, sgate, y)
+        return y

@@ -59,7 +59,7 @@ class HybridCacheManager:
     def __init__(self, n_pages: int, page_size: int, n_slots: int, kv_layers: Dict[int, Tuple[int, int, int]],
                  state_layers: Dict[int, Dict[str, Tuple[int, ...]]], dtype=torch.bfloat16, device="cuda",
                  max_tokens: int = 4096, max_rows: int = 32, max_step_tokens: int = 8192):
-        """kv_layers: layer run -> (kv_heads, key width, value width); state_layers: layer run ->
+        """kv_layers: layer run -> (kv_heads, key width, value width; 0 = no separate values); state_layers: layer run ->
         {name: shape per slot} (fp32).  `max_tokens`: the longest sequence a block-table row
         describes."""
         self.n_pages, self.page_size, self.n_slots = n_pages, page_size, n_slots
@@ -67,7 +67,8 @@ class HybridCacheManager:
         self.k_caches, self.v_caches, self.states = {}, {}, {}
         for li, (g, d, dv) in kv_layers.items():
             self.k_caches[li] = torch.zeros(n_pages, page_size, g, d, dtype=dtype, device=device)
-            self.v_caches[li] = torch.zeros(n_pages, page_size, g, dv, dtype=dtype, device=device)
+            # value width 0: what a token keeps serves as key and value alike (a cached latent)
+            self.v_caches[li] = torch.zeros(n_pages, page_size, g, dv, dtype=dtype, device=device) if dv else None
         for li, named in state_layers.items():
             self.states[li] = {name: torch.zeros((n_slots,) + tuple(shape), dtype=torch.float32, device=device)
                                for name, shape in named.items()}

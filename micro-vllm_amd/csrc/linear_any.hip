@@ -15,6 +15,14 @@ namespace mv {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 la_bf16x8_t;
 
+// Rows in segments: with `seg` the launch's z-th product owns output rows seg[z] .. seg[z+1] (tokens sorted by
+// the expert they go to) and reads, for output row i, operand row src[i] / src_div (src == NULL: row i).
+struct RowSegments {
+    const int* seg;
+    const int* src;
+    int src_div;
+};
+
 constexpr int kLaBM = 64, kLaBN = 64, kLaBK = 32, kLaPad = 40;  // LDS row = 40 bf16 = 80 bytes
 
 __device__ __forceinline__ uint4 la_load8(const uint16_t* base, int64_t ld, int row, int nrows, int col, int k,
@@ -31,12 +39,29 @@ __device__ __forceinline__ uint4 la_load8(const uint16_t* base, int64_t ld, int 
 
 __global__ __launch_bounds__(256) void linear_any_bf16_kernel(
     const uint16_t* __restrict__ x, int64_t ldx, const uint16_t* __restrict__ w, int64_t ldw,
-    float* __restrict__ y, int64_t ldy, int M, int N, int K, int vec_x, int vec_w) {
+    float* __restrict__ y, int64_t ldy, int M, int N, int K, int vec_x, int vec_w, int64_t zx, int64_t zw,
+    int64_t zy, RowSegments sg) {
+    x += blockIdx.z * zx;   // blockIdx.z: one of several products that share a launch (per-head weights)
+    w += blockIdx.z * zw;
+    y += blockIdx.z * zy;
     __shared__ __attribute__((aligned(16))) uint16_t xs[kLaBM][kLaPad];
     __shared__ __attribute__((aligned(16))) uint16_t ws[kLaBN][kLaPad];
     const int m0 = blockIdx.y * kLaBM, n0 = blockIdx.x * kLaBN;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, q = lane >> 4;
     const int lrow = tid >> 2, lcol = (tid & 3) * 8;
+    int64_t y0 = 0;
+    if (sg.seg) {   // blockIdx.z owns output rows seg[z] .. seg[z+1]
+        y0 = sg.seg[blockIdx.z];
+        M = sg.seg[blockIdx.z + 1] - (int)y0;
+        if (m0 >= M) return;
+        y += y0 * ldy;
+    }
+    // this thread's operand row: the output row itself, or the row the segment's list names for it
+    {
+        const int mr = m0 + lrow;
+        const int64_t xrow = mr < M ? (sg.src ? sg.src[y0 + mr] / sg.src_div : y0 + mr) : 0;
+        x += xrow * ldx - (int64_t)(m0 + lrow) * ldx;
+    }
     f32x4_t acc[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
     uint4 xr = la_load8(x, ldx, m0 + lrow, M, lcol, K, vec_x);
     uint4 wr = la_load8(w, ldw, n0 + lrow, N, lcol, K, vec_w);
@@ -74,12 +99,27 @@ constexpr int kLfBK = 16;
 
 __global__ __launch_bounds__(256) void linear_any_f32_kernel(
     const float* __restrict__ x, int64_t ldx, const float* __restrict__ w, int64_t ldw,
-    float* __restrict__ y, int64_t ldy, int M, int N, int K) {
+    float* __restrict__ y, int64_t ldy, int M, int N, int K, int64_t zx, int64_t zw, int64_t zy, RowSegments sg) {
+    x += blockIdx.z * zx;
+    w += blockIdx.z * zw;
+    y += blockIdx.z * zy;
     __shared__ float xs[kLfBK][kLaBM + 4];
     __shared__ float ws[kLfBK][kLaBN + 4];
     const int m0 = blockIdx.y * kLaBM, n0 = blockIdx.x * kLaBN;
     const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
     const int lrow = tid >> 2, lcol = (tid & 3) * 4;
+    int64_t y0 = 0;
+    if (sg.seg) {
+        y0 = sg.seg[blockIdx.z];
+        M = sg.seg[blockIdx.z + 1] - (int)y0;
+        if (m0 >= M) return;
+        y += y0 * ldy;
+    }
+    {
+        const int mr = m0 + lrow;
+        const int64_t xrow = mr < M ? (sg.src ? sg.src[y0 + mr] / sg.src_div : y0 + mr) : 0;
+        x += xrow * ldx - (int64_t)(m0 + lrow) * ldx;
+    }
     float acc[4][4] = {};
     for (int k0 = 0; k0 < K; k0 += kLfBK) {
         __syncthreads();
@@ -118,22 +158,50 @@ __global__ __launch_bounds__(256) void linear_any_f32_kernel(
 
 }  // namespace mv
 
-extern "C" int mv_linear_any(const void* x, int64_t ldx, const void* w, int64_t ldw, float* y, int64_t ldy,
-                             int m, int n, int k, int f32, mv_stream_t stream) {
+static int launch_linear_any(const void* x, int64_t ldx, const void* w, int64_t ldw, float* y, int64_t ldy, int m, int n,
+                             int k, int f32, int batch, int64_t zx, int64_t zw, int64_t zy, mv_stream_t stream,
+                             mv::RowSegments sg = mv::RowSegments{nullptr, nullptr, 1}) {
     using namespace mv;
-    if (m < 0 || n <= 0 || k <= 0) return MV_ERR_INVALID_ARG;
-    if (m == 0) return MV_OK;
-    if (!x || !w || !y || ldx < k || ldw < k || ldy < n) return MV_ERR_INVALID_ARG;
-    const dim3 grid((n + kLaBN - 1) / kLaBN, (m + kLaBM - 1) / kLaBM);
-    if (grid.y > 65535) return MV_ERR_UNSUPPORTED;
+    const dim3 grid((n + kLaBN - 1) / kLaBN, (m + kLaBM - 1) / kLaBM, batch);
+    if (grid.y > 65535 || batch > 65535) return MV_ERR_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
     if (f32) {
         hipLaunchKernelGGL(linear_any_f32_kernel, grid, dim3(256), 0, s, (const float*)x, ldx, (const float*)w, ldw,
-                           y, ldy, m, n, k);
+                           y, ldy, m, n, k, zx, zw, zy, sg);
     } else {
-        const int vx = aligned16(x) && ldx % 8 == 0, vw = aligned16(w) && ldw % 8 == 0;
+        const int vx = aligned16(x) && ldx % 8 == 0 && zx % 8 == 0, vw = aligned16(w) && ldw % 8 == 0 && zw % 8 == 0;
         hipLaunchKernelGGL(linear_any_bf16_kernel, grid, dim3(256), 0, s, (const uint16_t*)x, ldx, (const uint16_t*)w,
-                           ldw, y, ldy, m, n, k, vx, vw);
+                           ldw, y, ldy, m, n, k, vx, vw, zx, zw, zy, sg);
     }
     return check_launch();
+}
+
+extern "C" int mv_linear_any(const void* x, int64_t ldx, const void* w, int64_t ldw, float* y, int64_t ldy,
+                             int m, int n, int k, int f32, mv_stream_t stream) {
+    if (m < 0 || n <= 0 || k <= 0) return MV_ERR_INVALID_ARG;
+    if (m == 0) return MV_OK;
+    if (!x || !w || !y || ldx < k || ldw < k || ldy < n) return MV_ERR_INVALID_ARG;
+    return launch_linear_any(x, ldx, w, ldw, y, ldy, m, n, k, f32, 1, 0, 0, 0, stream);
+}
+
+// `heads` products in one launch: y[:, h*zy + ..n] = x[:, h*zx + ..k] . W_h^T with W_h = w + h*zw ([n,k], row stride ldw)
+extern "C" int mv_linear_heads(const void* x, int64_t ldx, int64_t zx, const void* w, int64_t ldw, int64_t zw, float* y,
+                               int64_t ldy, int64_t zy, int m, int n, int k, int heads, int f32, mv_stream_t stream) {
+    if (m < 0 || n <= 0 || k <= 0 || heads <= 0 || zx < 0 || zw < 0 || zy < 0) return MV_ERR_INVALID_ARG;
+    if (m == 0) return MV_OK;
+    if (!x || !w || !y || ldx < (heads - 1) * zx + k || ldw < k || ldy < (heads - 1) * zy + n) return MV_ERR_INVALID_ARG;
+    return launch_linear_any(x, ldx, w, ldw, y, ldy, m, n, k, f32, heads, zx, zw, zy, stream);
+}
+
+// Products by segment: output rows seg[e] .. seg[e+1] (e < segments) use weight w + e*zw; `max_rows` bounds the
+// rows of any one segment (the launch has that many row tiles per segment, the ones past a segment's end leave
+// at once).  src: operand row of output row i is src[i] / src_div (NULL: i).
+extern "C" int mv_linear_segments(const void* x, int64_t ldx, const void* w, int64_t ldw, int64_t zw, float* y,
+                                  int64_t ldy, const int32_t* seg, const int32_t* src, int src_div, int segments,
+                                  int max_rows, int n, int k, int f32, mv_stream_t stream) {
+    if (max_rows < 0 || n <= 0 || k <= 0 || segments <= 0 || src_div <= 0 || zw < 0) return MV_ERR_INVALID_ARG;
+    if (max_rows == 0) return MV_OK;
+    if (!x || !w || !y || !seg || ldx < k || ldw < k || ldy < n) return MV_ERR_INVALID_ARG;
+    return launch_linear_any(x, ldx, w, ldw, y, ldy, max_rows, n, k, f32, segments, 0, zw, 0, stream,
+                             mv::RowSegments{seg, src, src_div});
 }

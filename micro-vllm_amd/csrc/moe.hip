@@ -1,0 +1,159 @@
+// Routed feed-forward (mixture of experts) over a step's tokens, everything on the device so that a step
+// can be recorded into a graph:
+//
+//   moe_route    logits = W_router h in fp32 (h in the activation type), the `top` largest (ties: the lower
+//                index), weights = softmax over the chosen logits; beside it sigmoid(w_sg . h), the factor
+//                of a shared expert (one number per token)
+//   moe_plan     the step's T * top (token, choice) pairs sorted by expert: seg[e] .. seg[e+1] are expert e's
+//                rows, order[i] the pair (token * top + choice) in row i, place[pair] its row.  The order inside
+//                an expert is whatever the atomics give; no result depends on it, since a row's products do
+//                not depend on the other rows (mv_linear_segments)
+//   moe_combine  y_t = sum_k weight[t,k] * expert_out[place[t,k]] (+ factor_t * shared_out_t)
+// The experts' products themselves are mv_linear_segments (linear_any.hip) with a SiLU-gate between them.
+#include "common.h"
+
+namespace mv {
+
+constexpr int kMaxExperts = 1024, kMaxTop = 16;
+
+template <bool F32>
+__global__ __launch_bounds__(256) void moe_route_kernel(const void* h_, int64_t ldh, const float* wr, const float* wsg,
+                                                        int* ids, float* wts, float* shared_gate, int n, int E,
+                                                        int top) {
+    __shared__ float z[kMaxExperts + 1];
+    const int t = blockIdx.x, wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int units = E + (wsg ? 1 : 0);
+    for (int e = wv; e < units; e += 4) {
+        const float* w = e < E ? wr + (int64_t)e * n : wsg;
+        float dot = 0.f;
+        if (F32) {
+            const float* h = (const float*)h_ + (int64_t)t * ldh;
+            for (int c = lane; c < n; c += 64) dot = fmaf(h[c], w[c], dot);
+        } else {
+            const uint16_t* h = (const uint16_t*)h_ + (int64_t)t * ldh;
+            for (int c = lane; c < n; c += 64) dot = fmaf(bf16_bits_to_f32(h[c]), w[c], dot);
+        }
+        dot = wave_sum(dot);
+        if (lane == 0) z[e] = dot;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int pick[kMaxTop];
+        float val[kMaxTop];
+        for (int k = 0; k < top; ++k) {
+            int best = -1;
+            float bv = -INFINITY;
+            for (int e = 0; e < E; ++e) {
+                bool taken = false;
+                for (int j = 0; j < k; ++j) taken |= pick[j] == e;
+                if (!taken && (best < 0 || z[e] > bv)) {
+                    best = e;
+                    bv = z[e];
+                }
+            }
+            pick[k] = best;
+            val[k] = bv;
+        }
+        float sum = 0.f;
+        const float largest = val[0];
+        for (int k = 0; k < top; ++k) {
+            val[k] = expf(val[k] - largest);
+            sum += val[k];
+        }
+        for (int k = 0; k < top; ++k) {
+            ids[(int64_t)t * top + k] = pick[k];
+            wts[(int64_t)t * top + k] = val[k] / sum;
+        }
+        if (wsg) shared_gate[t] = 1.0f / (1.0f + expf(-z[E]));
+    }
+}
+
+__global__ __launch_bounds__(1024) void moe_plan_kernel(const int* ids, int* seg, int* order, int* place, int pairs,
+                                                        int E) {
+    __shared__ int cnt[kMaxExperts + 1];
+    __shared__ int cur[kMaxExperts];
+    for (int e = threadIdx.x; e <= E; e += 1024) cnt[e] = 0;
+    __syncthreads();
+    for (int i = threadIdx.x; i < pairs; i += 1024) atomicAdd(&cnt[ids[i]], 1);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int run = 0;
+        for (int e = 0; e < E; ++e) {
+            const int c = cnt[e];
+            cur[e] = run;
+            seg[e] = run;
+            run += c;
+        }
+        seg[E] = run;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < pairs; i += 1024) {
+        const int row = atomicAdd(&cur[ids[i]], 1);
+        order[row] = i;
+        place[i] = row;
+    }
+}
+
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* eo, int64_t lde, const int* place,
+                                                          const float* wts, const float* so, int64_t lds_,
+                                                          const float* shared_gate, float* y, int64_t ldy, int n,
+                                                          int top) {
+    const int t = blockIdx.x;
+    int rows[kMaxTop];
+    float w[kMaxTop];
+    for (int k = 0; k < top; ++k) {
+        rows[k] = place[(int64_t)t * top + k];
+        w[k] = wts[(int64_t)t * top + k];
+    }
+    const float g = so ? shared_gate[t] : 0.f;
+    for (int c = threadIdx.x; c < n; c += 256) {
+        float acc = 0.f;
+        for (int k = 0; k < top; ++k) acc = fmaf(w[k], eo[(int64_t)rows[k] * lde + c], acc);
+        if (so) acc = fmaf(g, so[(int64_t)t * lds_ + c], acc);
+        y[(int64_t)t * ldy + c] = acc;
+    }
+}
+
+}  // namespace mv
+
+extern "C" {
+
+int mv_moe_route(const void* h, int64_t ldh, const float* w_router, const float* w_shared_gate, int32_t* ids,
+                 float* weights, float* shared_gate, int tokens, int n, int experts, int top, int f32,
+                 mv_stream_t stream) {
+    using namespace mv;
+    if (tokens < 0 || n <= 0 || experts <= 0 || experts > kMaxExperts || top <= 0 || top > kMaxTop || top > experts)
+        return MV_ERR_INVALID_ARG;
+    if (tokens == 0) return MV_OK;
+    if (!h || !w_router || !ids || !weights || (w_shared_gate && !shared_gate) || ldh < n) return MV_ERR_INVALID_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    if (f32) hipLaunchKernelGGL(moe_route_kernel<true>, dim3(tokens), dim3(256), 0, s, h, ldh, w_router, w_shared_gate, ids, weights, shared_gate, n, experts, top);
+    else hipLaunchKernelGGL(moe_route_kernel<false>, dim3(tokens), dim3(256), 0, s, h, ldh, w_router, w_shared_gate, ids, weights, shared_gate, n, experts, top);
+    return check_launch();
+}
+
+int mv_moe_plan(const int32_t* ids, int32_t* seg, int32_t* order, int32_t* place, int pairs, int experts,
+                mv_stream_t stream) {
+    using namespace mv;
+    if (pairs < 0 || experts <= 0 || experts > kMaxExperts) return MV_ERR_INVALID_ARG;
+    if (!ids || !seg || !order || !place) return MV_ERR_INVALID_ARG;
+    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, ids, seg, order, place, pairs,
+                       experts);
+    return check_launch();
+}
+
+int mv_moe_combine(const float* expert_out, int64_t lde, const int32_t* place, const float* weights,
+                   const float* shared_out, int64_t lds, const float* shared_gate, float* y, int64_t ldy, int tokens,
+                   int n, int top, mv_stream_t stream) {
+    using namespace mv;
+    if (tokens < 0 || n <= 0 || top <= 0 || top > kMaxTop) return MV_ERR_INVALID_ARG;
+    if (tokens == 0) return MV_OK;
+    if (!expert_out || !place || !weights || !y || (shared_out && !shared_gate) || lde < n || ldy < n ||
+        (shared_out && lds < n))
+        return MV_ERR_INVALID_ARG;
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(tokens), dim3(256), 0, (hipStream_t)stream, expert_out, lde, place,
+                       weights, shared_out, lds, shared_gate, y, ldy, n, top);
+    return check_launch();
+}
+
+}  // extern "C"

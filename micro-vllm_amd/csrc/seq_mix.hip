@@ -8,6 +8,9 @@
 //   softplus_decay                 step sizes and decays of a selective state-space head
 //   scan_outer                     S_t = decay_t S_(t-1) + gain_t k_t v_t^T,  o_t = S_t^T q_t (+ skip_h v_t)
 //                                  (state-space duality heads and fixed-decay retention heads alike)
+//   scan_gated                     S_t = diag(f_t) S_(t-1) + (1 - f_t) v_t^T,  o_t = S_t^T q_t: a forget gate per
+//                                  state row that also scales what is written (no key)
+//   gate_lower_bound               q = silu(q), f = l + (1 - l) sigmoid(f + b) in place, ahead of scan_gated
 //   rotary_pairs                   rotate-half rotation of the first `rot` dimensions of each head
 //   gated_group_norm               unit-RMS per group with a SiLU gate before or after it
 //   qk_unitnorm_store              per-head unit-RMS of queries and keys, keys/values into their pages
@@ -106,7 +109,8 @@ struct ScanArgs {
     int max_len;   // rows longer than this belong to the chunked form (0: every row is taken)
 };
 
-template <int MAXN>
+// GATED: `decay` holds a forget gate per (token, head, state row) and the key is one minus it.
+template <int MAXN, bool GATED = false>
 __global__ __launch_bounds__(256) void scan_outer_kernel(ScanArgs a) {
     __shared__ float part[2][256];
     const int b = blockIdx.z, h = blockIdx.y, tid = threadIdx.x;
@@ -123,18 +127,30 @@ __global__ __launch_bounds__(256) void scan_outer_kernel(ScanArgs a) {
     for (int i = 0; i < MAXN; ++i) S[i] = (carried && vc && i < npt && n0 + i < a.n) ? sp[(int64_t)i * a.p] : 0.f;
     for (int t = 0; t < len; ++t) {
         const int64_t tok = start + t;
-        const float dec = a.decay[tok * a.ld_decay + h];
-        const float g = a.gain ? a.gain[tok * a.ld_gain + h] : 1.0f;
         const float vv = vc ? a.v[tok * a.ldv + (int64_t)h * a.p + c] : 0.f;
-        const float gv = g * vv;
-        const float* kp = a.k + tok * a.ldk + (int64_t)(h / a.k_div) * a.n + n0;
         const float* qp = a.q + tok * a.ldq + (int64_t)(h / a.q_div) * a.n + n0;
         float o = 0.f;
+        if (GATED) {
+            const float* fp = a.decay + tok * a.ld_decay + (int64_t)h * a.n + n0;
 #pragma unroll
-        for (int i = 0; i < MAXN; ++i) {
-            if (i < npt && n0 + i < a.n) {
-                S[i] = fmaf(kp[i], gv, dec * S[i]);
-                o = fmaf(S[i], qp[i], o);
+            for (int i = 0; i < MAXN; ++i) {
+                if (i < npt && n0 + i < a.n) {
+                    const float f = fp[i];
+                    S[i] = fmaf(1.0f - f, vv, f * S[i]);
+                    o = fmaf(S[i], qp[i], o);
+                }
+            }
+        } else {
+            const float dec = a.decay[tok * a.ld_decay + h];
+            const float g = a.gain ? a.gain[tok * a.ld_gain + h] : 1.0f;
+            const float gv = g * vv;
+            const float* kp = a.k + tok * a.ldk + (int64_t)(h / a.k_div) * a.n + n0;
+#pragma unroll
+            for (int i = 0; i < MAXN; ++i) {
+                if (i < npt && n0 + i < a.n) {
+                    S[i] = fmaf(kp[i], gv, dec * S[i]);
+                    o = fmaf(S[i], qp[i], o);
+                }
             }
         }
         part[t & 1][tid] = o;
@@ -378,6 +394,18 @@ __global__ __launch_bounds__(256) void scan_chunk_inter_kernel(ChunkArgs a) {
             }
         }
     }
+}
+
+__global__ __launch_bounds__(256) void gate_lower_bound_kernel(float* q, int64_t ldq, float* f, int64_t ldf,
+                                                               const float* bias, const float* lower, int T, int n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (int64_t)T * n) return;
+    const int t = (int)(i / n), c = (int)(i % n);
+    float* qp = q + (int64_t)t * ldq + c;
+    float* fp = f + (int64_t)t * ldf + c;
+    *qp = silu_f(*qp);
+    const float l = lower[c], z = *fp + (bias ? bias[c] : 0.f);
+    *fp = fmaf(1.0f - l, 1.0f / (1.0f + expf(-z)), l);
 }
 
 __global__ __launch_bounds__(256) void rotary_pairs_kernel(float* x, int64_t ld, const double* inv_freq,
@@ -801,10 +829,49 @@ int mv_scan_outer(const float* q, int64_t ldq, int q_div, const float* k, int64_
     const int ns = 256 / a.pt, npt = (n + ns - 1) / ns;
     const dim3 grid((p + a.pt - 1) / a.pt, heads, rows);
     hipStream_t s = (hipStream_t)stream;
-    if (npt <= 4) hipLaunchKernelGGL(scan_outer_kernel<4>, grid, dim3(256), 0, s, a);
-    else if (npt <= 16) hipLaunchKernelGGL(scan_outer_kernel<16>, grid, dim3(256), 0, s, a);
-    else if (npt <= 64) hipLaunchKernelGGL(scan_outer_kernel<64>, grid, dim3(256), 0, s, a);
+    if (npt <= 4) hipLaunchKernelGGL((scan_outer_kernel<4, false>), grid, dim3(256), 0, s, a);
+    else if (npt <= 16) hipLaunchKernelGGL((scan_outer_kernel<16, false>), grid, dim3(256), 0, s, a);
+    else if (npt <= 64) hipLaunchKernelGGL((scan_outer_kernel<64, false>), grid, dim3(256), 0, s, a);
     else return MV_ERR_UNSUPPORTED;
+    return check_launch();
+}
+
+int mv_scan_gated(const float* q, int64_t ldq, const float* f, int64_t ldf, const float* v, int64_t ldv, float* state,
+                  float* out, int64_t ldo, const int32_t* row_start, const int32_t* row_len, const int32_t* row_ctx,
+                  const int32_t* row_slot, int rows, int heads, int n, int p, mv_stream_t stream) {
+    using namespace mv;
+    if (rows < 0 || heads <= 0 || n <= 0 || p <= 0) return MV_ERR_INVALID_ARG;
+    if (rows == 0) return MV_OK;
+    if (!q || !f || !v || !state || !out || rows > 65535 || heads > 65535) return MV_ERR_INVALID_ARG;
+    if (ldq < (int64_t)heads * n || ldf < (int64_t)heads * n || ldv < (int64_t)heads * p || ldo < (int64_t)heads * p)
+        return MV_ERR_INVALID_ARG;
+    ScanArgs a;
+    a.q = q; a.k = nullptr; a.v = v; a.decay = f; a.gain = nullptr; a.skip = nullptr;
+    a.ldq = ldq; a.ldk = 0; a.ldv = ldv; a.ld_decay = ldf; a.ld_gain = 0; a.ldo = ldo;
+    a.q_div = 1; a.k_div = 1; a.state = state; a.out = out;
+    a.r = StepRows{nullptr, nullptr, row_start, row_len, row_ctx, row_slot};
+    a.H = heads; a.n = n; a.p = p; a.max_len = 0;
+    a.pt = p % 64 == 0 ? 64 : (p % 32 == 0 ? 32 : 16);
+    while (a.pt > 16 && (n + 256 / a.pt - 1) / (256 / a.pt) > 64) a.pt /= 2;
+    const int ns = 256 / a.pt, npt = (n + ns - 1) / ns;
+    const dim3 grid((p + a.pt - 1) / a.pt, heads, rows);
+    hipStream_t s = (hipStream_t)stream;
+    if (npt <= 4) hipLaunchKernelGGL((scan_outer_kernel<4, true>), grid, dim3(256), 0, s, a);
+    else if (npt <= 16) hipLaunchKernelGGL((scan_outer_kernel<16, true>), grid, dim3(256), 0, s, a);
+    else if (npt <= 64) hipLaunchKernelGGL((scan_outer_kernel<64, true>), grid, dim3(256), 0, s, a);
+    else return MV_ERR_UNSUPPORTED;
+    return check_launch();
+}
+
+int mv_gate_lower_bound(float* q, int64_t ldq, float* f, int64_t ldf, const float* bias, const float* lower,
+                        int tokens, int n, mv_stream_t stream) {
+    using namespace mv;
+    if (tokens < 0 || n <= 0) return MV_ERR_INVALID_ARG;
+    if (tokens == 0) return MV_OK;
+    if (!q || !f || !lower || ldq < n || ldf < n) return MV_ERR_INVALID_ARG;
+    const int64_t total = (int64_t)tokens * n;
+    hipLaunchKernelGGL(gate_lower_bound_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, q, ldq, f, ldf, bias, lower, tokens, n);
     return check_launch();
 }
 

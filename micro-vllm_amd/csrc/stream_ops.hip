@@ -9,6 +9,15 @@
 //   offset_rmsnorm_gather: out = act( x[idx] / sqrt(mean(x[idx]^2) + eps) * (1 + w) )
 //   relu_squared:        out = act( max(v, 0)^2 )
 //   softcap:             v = cap * tanh(v / cap)
+//   dyt_shift:           n = tanh(alpha x) w + b (a norm without statistics); h_t = act( n_t + (n_(t-1) - n_t) mix ),
+//                        the last n of every row kept per state slot for the row's next step
+//   dyt_gather:          out = act( tanh(alpha x[idx]) w + b )
+//   dyt_residual:        x += tanh(alpha y) w + b; h = act(x)
+//   unitnorm_residual:   x += y / sqrt(mean(y^2) + eps) * w; h = act(x)     (plain weight)
+//   rmsnorm_rows:        out = act( v / sqrt(mean(v^2) + eps) * w )         (plain weight, rows of any stride)
+//   gelu_gate_rows:      out = act( gelu_tanh(a) * table[id][off .. off+n) )
+//   silu_mul:            out = act( silu(a[:, :n]) * a[:, n:2n] )
+//   sigmoid_gate:        out = act( a * sigmoid(g) )   (g == NULL: act(a))
 // All arithmetic is fp32 with the library's exact division, square root and tanh.
 #include "common.h"
 
@@ -101,6 +110,147 @@ __global__ __launch_bounds__(256) void softcap_kernel(float* v, int64_t count, f
     if (i < count) v[i] = cap * tanhf(v[i] / cap);
 }
 
+// ---- Dynamic Tanh norm, token shift ------------------------------------------------------------------
+// One workgroup per token.  n_(t-1) of a row's first token is the slot's kept vector (zeros when the
+// sequence holds nothing yet); the workgroup of that first token also writes the row's LAST n into the
+// slot, so that nobody else touches the slot in this launch.
+template <bool F32>
+__global__ __launch_bounds__(256) void dyt_shift_kernel(const float* x, int64_t ldx, const float* w, const float* b,
+                                                        const float* alpha, const float* mix, float* state,
+                                                        void* h_, int64_t ldh, const int* tok_row,
+                                                        const int* row_start, const int* row_len, const int* row_ctx,
+                                                        const int* row_slot, int n) {
+    typedef typename Act<F32>::T T;
+    T* h = (T*)h_;
+    const int t = blockIdx.x, r = tok_row[t];
+    const int first = row_start[r], len = row_len[r];
+    const float al = alpha[0];
+    const float* cur = x + (int64_t)t * ldx;
+    const bool head = t == first;
+    float* kept = state + (int64_t)row_slot[r] * n;
+    const bool carried = row_ctx[r] > 0;
+    const float* prev = x + (int64_t)(t - 1) * ldx;
+    const float* last = x + (int64_t)(first + len - 1) * ldx;
+    for (int c = threadIdx.x; c < n; c += 256) {
+        const float nc = fmaf(tanhf(al * cur[c]), w[c], b[c]);
+        float np;
+        if (head) np = carried ? kept[c] : 0.f;
+        else np = fmaf(tanhf(al * prev[c]), w[c], b[c]);
+        Act<F32>::st(h + (int64_t)t * ldh + c, fmaf(np - nc, mix[c], nc));
+        if (head) kept[c] = len == 1 ? nc : fmaf(tanhf(al * last[c]), w[c], b[c]);
+    }
+}
+
+template <bool F32>
+__global__ __launch_bounds__(256) void dyt_gather_kernel(const float* x, int64_t ldx, const int* idx, const float* w,
+                                                         const float* b, const float* alpha, void* out_, int64_t ldo,
+                                                         int n) {
+    typedef typename Act<F32>::T T;
+    T* out = (T*)out_;
+    const int row = blockIdx.x;
+    const float* a = x + (int64_t)(idx ? idx[row] : row) * ldx;
+    const float al = alpha[0];
+    for (int c = threadIdx.x; c < n; c += 256)
+        Act<F32>::st(out + (int64_t)row * ldo + c, fmaf(tanhf(al * a[c]), w[c], b[c]));
+}
+
+template <bool F32>
+__global__ __launch_bounds__(256) void dyt_residual_kernel(const float* y, int64_t ldy, const float* w, const float* b,
+                                                           const float* alpha, float* x, int64_t ldx, void* h_,
+                                                           int64_t ldh, int n) {
+    typedef typename Act<F32>::T T;
+    T* h = (T*)h_;
+    const int row = blockIdx.x;
+    const float al = alpha[0];
+    for (int c = threadIdx.x; c < n; c += 256) {
+        const float s = x[(int64_t)row * ldx + c] + fmaf(tanhf(al * y[(int64_t)row * ldy + c]), w[c], b[c]);
+        x[(int64_t)row * ldx + c] = s;
+        if (h) Act<F32>::st(h + (int64_t)row * ldh + c, s);
+    }
+}
+
+template <bool F32>
+__global__ __launch_bounds__(256) void unitnorm_residual_kernel(const float* y, int64_t ldy, const float* w, float eps,
+                                                                float* x, int64_t ldx, void* h_, int64_t ldh, int n) {
+    typedef typename Act<F32>::T T;
+    __shared__ float red[4];
+    T* h = (T*)h_;
+    const int row = blockIdx.x;
+    const float* a = y + (int64_t)row * ldy;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < n; c += 256) ss += a[c] * a[c];
+    ss = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+    for (int c = threadIdx.x; c < n; c += 256) {
+        const float s = x[(int64_t)row * ldx + c] + (a[c] * inv) * w[c];
+        x[(int64_t)row * ldx + c] = s;
+        if (h) Act<F32>::st(h + (int64_t)row * ldh + c, s);
+    }
+}
+
+// one wave per row of `n` values (rows may be heads of a wider buffer: row r starts at (r / per) * ld + (r % per) * n)
+template <bool F32>
+__global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const float* v, int64_t ld, int per, const float* w,
+                                                           float eps, void* out_, int64_t ldo, int64_t rows, int n) {
+    typedef typename Act<F32>::T T;
+    T* out = (T*)out_;
+    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (r >= rows) return;
+    const float* a = v + (r / per) * ld + (r % per) * n;
+    T* o = out + (r / per) * ldo + (r % per) * n;
+    float ss = 0.f;
+    for (int c = lane; c < n; c += 64) ss += a[c] * a[c];
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+    for (int c = lane; c < n; c += 64) Act<F32>::st(o + c, (a[c] * inv) * w[c]);
+}
+
+__device__ __forceinline__ float gelu_tanh_f(float z) {
+    const float inner = 0.7978845608028654f * fmaf(0.044715f * z * z, z, z);
+    return 0.5f * z * (1.0f + tanhf(inner));
+}
+
+template <bool F32>
+__global__ __launch_bounds__(256) void gelu_gate_rows_kernel(const float* a, int64_t lda, const void* table_,
+                                                             int64_t ldt, int off, const int* ids, int vocab,
+                                                             void* out_, int64_t ldo, int n) {
+    typedef typename Act<F32>::T T;
+    const T* table = (const T*)table_;
+    T* out = (T*)out_;
+    const int row = blockIdx.x;
+    int id = ids[row];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+    for (int c = threadIdx.x; c < n; c += 256) {
+        const float e = Act<F32>::ld(table + (int64_t)id * ldt + off + c);
+        Act<F32>::st(out + (int64_t)row * ldo + c, gelu_tanh_f(a[(int64_t)row * lda + c]) * e);
+    }
+}
+
+template <bool F32>
+__global__ __launch_bounds__(256) void silu_mul_kernel(const float* a, int64_t lda, void* out_, int64_t ldo, int n) {
+    typedef typename Act<F32>::T T;
+    T* out = (T*)out_;
+    const int64_t row = blockIdx.x;
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= n) return;
+    const float g = a[row * lda + c], u = a[row * lda + n + c];
+    Act<F32>::st(out + row * ldo + c, (g / (1.0f + expf(-g))) * u);
+}
+
+template <bool F32>
+__global__ __launch_bounds__(256) void sigmoid_gate_kernel(const float* a, int64_t lda, const float* g, int64_t ldg,
+                                                           void* out_, int64_t ldo, int n) {
+    typedef typename Act<F32>::T T;
+    T* out = (T*)out_;
+    const int64_t row = blockIdx.x;
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= n) return;
+    float v = a[row * lda + c];
+    if (g) v = v / (1.0f + expf(-g[row * ldg + c]));
+    Act<F32>::st(out + row * ldo + c, v);
+}
+
 }  // namespace mv
 
 extern "C" {
@@ -161,6 +311,107 @@ int mv_softcap(float* v, int64_t count, float cap, mv_stream_t stream) {
     if (count == 0) return MV_OK;
     if (!v) return MV_ERR_INVALID_ARG;
     hipLaunchKernelGGL(softcap_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, (hipStream_t)stream, v, count, cap);
+    return check_launch();
+}
+
+#define MV_F32_LAUNCH(kern, grid, ...)                                                              \
+    do {                                                                                            \
+        if (f32) hipLaunchKernelGGL(kern<true>, grid, dim3(256), 0, s, __VA_ARGS__);                \
+        else hipLaunchKernelGGL(kern<false>, grid, dim3(256), 0, s, __VA_ARGS__);                   \
+    } while (0)
+
+int mv_dyt_shift(const float* x, int64_t ldx, const float* w, const float* b, const float* alpha, const float* mix,
+                 float* state, void* h, int64_t ldh, const int32_t* tok_row, const int32_t* row_start,
+                 const int32_t* row_len, const int32_t* row_ctx, const int32_t* row_slot, int tokens, int n, int f32,
+                 mv_stream_t stream) {
+    using namespace mv;
+    if (tokens < 0 || n <= 0) return MV_ERR_INVALID_ARG;
+    if (tokens == 0) return MV_OK;
+    if (!x || !w || !b || !alpha || !mix || !state || !h || !tok_row || !row_start || !row_len || !row_ctx ||
+        !row_slot || ldx < n || ldh < n)
+        return MV_ERR_INVALID_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    MV_F32_LAUNCH(dyt_shift_kernel, dim3(tokens), x, ldx, w, b, alpha, mix, state, h, ldh, tok_row, row_start, row_len,
+                  row_ctx, row_slot, n);
+    return check_launch();
+}
+
+int mv_dyt_gather(const float* x, int64_t ldx, const int32_t* idx, const float* w, const float* b, const float* alpha,
+                  void* out, int64_t ldo, int rows, int n, int f32, mv_stream_t stream) {
+    using namespace mv;
+    if (rows < 0 || n <= 0) return MV_ERR_INVALID_ARG;
+    if (rows == 0) return MV_OK;
+    if (!x || !w || !b || !alpha || !out || ldx < n || ldo < n) return MV_ERR_INVALID_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    MV_F32_LAUNCH(dyt_gather_kernel, dim3(rows), x, ldx, idx, w, b, alpha, out, ldo, n);
+    return check_launch();
+}
+
+int mv_dyt_residual(const float* y, int64_t ldy, const float* w, const float* b, const float* alpha, float* x,
+                    int64_t ldx, void* h, int64_t ldh, int rows, int n, int f32, mv_stream_t stream) {
+    using namespace mv;
+    if (rows < 0 || n <= 0) return MV_ERR_INVALID_ARG;
+    if (rows == 0) return MV_OK;
+    if (!y || !w || !b || !alpha || !x || ldy < n || ldx < n || (h && ldh < n)) return MV_ERR_INVALID_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    MV_F32_LAUNCH(dyt_residual_kernel, dim3(rows), y, ldy, w, b, alpha, x, ldx, h, ldh, n);
+    return check_launch();
+}
+
+int mv_unitnorm_residual(const float* y, int64_t ldy, const float* w, float eps, float* x, int64_t ldx, void* h,
+                         int64_t ldh, int rows, int n, int f32, mv_stream_t stream) {
+    using namespace mv;
+    if (rows < 0 || n <= 0) return MV_ERR_INVALID_ARG;
+    if (rows == 0) return MV_OK;
+    if (!y || !w || !x || ldy < n || ldx < n || (h && ldh < n)) return MV_ERR_INVALID_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    MV_F32_LAUNCH(unitnorm_residual_kernel, dim3(rows), y, ldy, w, eps, x, ldx, h, ldh, n);
+    return check_launch();
+}
+
+int mv_rmsnorm_rows(const float* v, int64_t ld, int per, const float* w, float eps, void* out, int64_t ldo,
+                    int rows, int n, int f32, mv_stream_t stream) {
+    using namespace mv;
+    if (rows < 0 || n <= 0 || per <= 0) return MV_ERR_INVALID_ARG;
+    if (rows == 0) return MV_OK;
+    if (!v || !w || !out || ld < (int64_t)per * n || ldo < (int64_t)per * n) return MV_ERR_INVALID_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    const int64_t total = (int64_t)rows * per;
+    MV_F32_LAUNCH(rmsnorm_rows_kernel, dim3((unsigned)((total + 3) / 4)), v, ld, per, w, eps, out, ldo, total, n);
+    return check_launch();
+}
+
+int mv_gelu_gate_rows(const float* a, int64_t lda, const void* table, int64_t ldt, int off, const int32_t* ids,
+                      int vocab, void* out, int64_t ldo, int rows, int n, int f32, mv_stream_t stream) {
+    using namespace mv;
+    if (rows < 0 || n <= 0 || vocab <= 0 || off < 0) return MV_ERR_INVALID_ARG;
+    if (rows == 0) return MV_OK;
+    if (!a || !table || !ids || !out || lda < n || ldt < off + n || ldo < n) return MV_ERR_INVALID_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    MV_F32_LAUNCH(gelu_gate_rows_kernel, dim3(rows), a, lda, table, ldt, off, ids, vocab, out, ldo, n);
+    return check_launch();
+}
+
+int mv_silu_mul(const float* a, int64_t lda, void* out, int64_t ldo, int rows, int n, int f32, mv_stream_t stream) {
+    using namespace mv;
+    if (rows < 0 || n <= 0) return MV_ERR_INVALID_ARG;
+    if (rows == 0) return MV_OK;
+    if (!a || !out || lda < 2 * (int64_t)n || ldo < n) return MV_ERR_INVALID_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid(rows, (n + 255) / 256);
+    MV_F32_LAUNCH(silu_mul_kernel, grid, a, lda, out, ldo, n);
+    return check_launch();
+}
+
+int mv_sigmoid_gate(const float* a, int64_t lda, const float* g, int64_t ldg, void* out, int64_t ldo, int rows, int n,
+                    int f32, mv_stream_t stream) {
+    using namespace mv;
+    if (rows < 0 || n <= 0) return MV_ERR_INVALID_ARG;
+    if (rows == 0) return MV_OK;
+    if (!a || !out || lda < n || (g && ldg < n) || ldo < n) return MV_ERR_INVALID_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid(rows, (n + 255) / 256);
+    MV_F32_LAUNCH(sigmoid_gate_kernel, grid, a, lda, g, ldg, out, ldo, n);
     return check_launch();
 }
 

@@ -237,3 +237,211 @@ def window_attn(q, k_cache, v_cache, out, step, slopes, heads: int, kv_heads: in
         int(window), _is_f32(k_cache), step.row_len.data_ptr(),
         step.ch_start.data_ptr() if step.n_chunks else None, step.ch_len.data_ptr() if step.n_chunks else None,
         step.n_chunks if tiled else 0, SCAN_SEQ_MAX, nv.stream_ptr()))
+
+
+# ---------------------------------------------------------------------------------------------------------
+# Dynamic Tanh norms, token shift, gated recurrence without a key, attention over a cached latent, routed
+# experts (csrc/stream_ops.hip, seq_mix.hip, latent_attn.hip, moe.hip, linear_any.hip)
+
+def _dyt(norm):
+    w, b, alpha = norm
+    assert w.is_contiguous() and b.is_contiguous() and w.numel() == b.numel() and alpha.numel() == 1
+    return _f32(w).data_ptr(), _f32(b).data_ptr(), _f32(alpha).data_ptr()
+
+
+def dyt_shift(x, norm, mix, state, h, step):
+    """h_t = act(n_t + (n_(t-1) - n_t) * mix) with n = tanh(alpha x) w + b; state [slots, n] keeps each row's
+    last n for its next step."""
+    tokens, n = x.shape
+    assert h.shape == (tokens, n) and norm[0].numel() == n and mix.numel() == n and mix.is_contiguous()
+    assert state.is_contiguous() and state.shape[1:] == (n,) and int(step.max_slot) < state.shape[0]
+    assert step.tokens == tokens
+    w, b, a = _dyt(norm)
+    nv.check("mv_dyt_shift", nv.lib().mv_dyt_shift(
+        _f32(x).data_ptr(), _ld(x), w, b, a, _f32(mix).data_ptr(), _f32(state).data_ptr(), h.data_ptr(), _ld(h),
+        step.tok_row.data_ptr(), step.row_start.data_ptr(), step.row_len.data_ptr(), step.row_ctx.data_ptr(),
+        step.row_slot.data_ptr(), tokens, n, _is_f32(h), nv.stream_ptr()))
+
+
+def dyt_gather(x, idx, norm, out):
+    rows, n = out.shape
+    assert x.shape[1] == n and norm[0].numel() == n and (idx is None or idx.numel() == rows)
+    assert idx is not None or x.shape[0] == rows
+    w, b, a = _dyt(norm)
+    nv.check("mv_dyt_gather", nv.lib().mv_dyt_gather(
+        _f32(x).data_ptr(), _ld(x), None if idx is None else _i32(idx).data_ptr(), w, b, a, out.data_ptr(), _ld(out),
+        rows, n, _is_f32(out), nv.stream_ptr()))
+
+
+def dyt_residual(y, norm, x, h=None, f32: bool = False):
+    """x += tanh(alpha y) w + b; h (optional) = x in the activation type."""
+    rows, n = x.shape
+    assert y.shape == (rows, n) and norm[0].numel() == n and (h is None or h.shape == (rows, n))
+    w, b, a = _dyt(norm)
+    nv.check("mv_dyt_residual", nv.lib().mv_dyt_residual(
+        _f32(y).data_ptr(), _ld(y), w, b, a, _f32(x).data_ptr(), _ld(x), None if h is None else h.data_ptr(),
+        0 if h is None else _ld(h), rows, n, int(f32) if h is None else _is_f32(h), nv.stream_ptr()))
+
+
+def unitnorm_residual(y, w, eps: float, x, h=None):
+    """x += y / sqrt(mean(y^2) + eps) * w; h (optional) = x in the activation type."""
+    rows, n = x.shape
+    assert y.shape == (rows, n) and w.numel() == n and w.is_contiguous() and (h is None or h.shape == (rows, n))
+    nv.check("mv_unitnorm_residual", nv.lib().mv_unitnorm_residual(
+        _f32(y).data_ptr(), _ld(y), _f32(w).data_ptr(), float(eps), _f32(x).data_ptr(), _ld(x),
+        None if h is None else h.data_ptr(), 0 if h is None else _ld(h), rows, n, 0 if h is None else _is_f32(h),
+        nv.stream_ptr()))
+
+
+def rmsnorm_rows(v, w, eps: float, out, per: int = 1):
+    """Each row of v holds `per` groups of w.numel() values: out = act(unit-RMS(group) * w)."""
+    rows, n = v.shape[0], w.numel()
+    assert v.shape[1] == per * n and out.shape == (rows, per * n) and w.is_contiguous()
+    nv.check("mv_rmsnorm_rows", nv.lib().mv_rmsnorm_rows(
+        _f32(v).data_ptr(), _ld(v), per, _f32(w).data_ptr(), float(eps), out.data_ptr(), _ld(out), rows, n,
+        _is_f32(out), nv.stream_ptr()))
+
+
+def gelu_gate_rows(a, table, off: int, ids, out):
+    rows, n = a.shape
+    assert out.shape == (rows, n) and table.is_cuda and table.dim() == 2 and table.stride(1) == 1
+    assert table.dtype == out.dtype and off + n <= table.shape[1] and ids.numel() == rows
+    nv.check("mv_gelu_gate_rows", nv.lib().mv_gelu_gate_rows(
+        _f32(a).data_ptr(), _ld(a), table.data_ptr(), table.stride(0), off, _i32(ids).data_ptr(), table.shape[0],
+        out.data_ptr(), _ld(out), rows, n, _is_f32(out), nv.stream_ptr()))
+
+
+def silu_mul(a, out):
+    rows, n = out.shape
+    assert a.shape == (rows, 2 * n)
+    nv.check("mv_silu_mul", nv.lib().mv_silu_mul(
+        _f32(a).data_ptr(), _ld(a), out.data_ptr(), _ld(out), rows, n, _is_f32(out), nv.stream_ptr()))
+
+
+def sigmoid_gate(a, g, out):
+    rows, n = a.shape
+    assert out.shape == (rows, n) and (g is None or g.shape == (rows, n))
+    nv.check("mv_sigmoid_gate", nv.lib().mv_sigmoid_gate(
+        _f32(a).data_ptr(), _ld(a), None if g is None else _f32(g).data_ptr(), 0 if g is None else _ld(g),
+        out.data_ptr(), _ld(out), rows, n, _is_f32(out), nv.stream_ptr()))
+
+
+def linear_heads(x, w, out, heads: int):
+    """out[:, h*n : (h+1)*n] = x[:, h*k : (h+1)*k] . w[h]^T for w [heads, n, k] in the activation type; fp32 out.
+    `out` may be a strided view [T, heads, n] of a wider buffer (row stride and head stride are passed on)."""
+    m = x.shape[0]
+    _, n, k = w.shape
+    assert w.is_cuda and w.is_contiguous() and w.shape[0] == heads and x.dtype == w.dtype
+    assert x.shape == (m, heads * k) and x.stride(1) == 1
+    assert out.dim() == 3 and out.shape == (m, heads, n) and out.stride(2) == 1 and out.dtype == torch.float32
+    if m == 0:
+        return out
+    ldy = out.stride(0) if m > 1 else max(out.stride(0), (heads - 1) * out.stride(1) + n)
+    nv.check("mv_linear_heads", nv.lib().mv_linear_heads(
+        x.data_ptr(), _ld(x), k, w.data_ptr(), k, n * k, out.data_ptr(), ldy, out.stride(1), m, n, k, heads,
+        _is_f32(x), nv.stream_ptr()))
+    return out
+
+
+def linear_segments(x, w, out, seg, src, src_div: int, max_rows: int):
+    """Rows seg[e] .. seg[e+1] of out = (operand rows src[i] // src_div, or i itself) . w[e]^T; w [E, n, k]."""
+    E, n, k = w.shape
+    assert w.is_cuda and w.is_contiguous() and x.dtype == w.dtype and x.shape[1] == k and x.stride(1) == 1
+    assert out.shape[1] == n and out.dtype == torch.float32 and out.stride(1) == 1 and seg.numel() == E + 1
+    assert src is None or src.numel() == out.shape[0]
+    assert src is not None or x.shape[0] == out.shape[0]
+    if out.shape[0] == 0:
+        return out
+    nv.check("mv_linear_segments", nv.lib().mv_linear_segments(
+        x.data_ptr(), _ld(x), w.data_ptr(), k, n * k, out.data_ptr(), _ld(out), _i32(seg).data_ptr(),
+        None if src is None else _i32(src).data_ptr(), src_div, E, min(max_rows, out.shape[0]), n, k, _is_f32(x),
+        nv.stream_ptr()))
+    return out
+
+
+def gate_lower_bound_(q, f, bias, lower):
+    tokens, n = q.shape
+    assert f.shape == (tokens, n) and lower.numel() == n and lower.is_contiguous()
+    assert bias is None or (bias.numel() == n and bias.is_contiguous())
+    nv.check("mv_gate_lower_bound", nv.lib().mv_gate_lower_bound(
+        _f32(q).data_ptr(), _ld(q), _f32(f).data_ptr(), _ld(f), None if bias is None else _f32(bias).data_ptr(),
+        _f32(lower).data_ptr(), tokens, n, nv.stream_ptr()))
+
+
+def scan_gated(q, f, v, state, out, step, heads: int, n: int, p: int):
+    """S_t = diag(f_t) S_(t-1) + (1 - f_t) v_t^T, o_t = S_t^T q_t; state [slots, heads, n, p] fp32."""
+    tokens = v.shape[0]
+    assert q.shape == (tokens, heads * n) and f.shape == (tokens, heads * n)
+    assert v.shape == (tokens, heads * p) and out.shape == (tokens, heads * p)
+    assert state.is_contiguous() and state.shape[1:] == (heads, n, p) and int(step.max_slot) < state.shape[0]
+    assert step.tokens == tokens
+    nv.check("mv_scan_gated", nv.lib().mv_scan_gated(
+        _f32(q).data_ptr(), _ld(q), _f32(f).data_ptr(), _ld(f), _f32(v).data_ptr(), _ld(v), _f32(state).data_ptr(),
+        _f32(out).data_ptr(), _ld(out), step.row_start.data_ptr(), step.row_len.data_ptr(), step.row_ctx.data_ptr(),
+        step.row_slot.data_ptr(), step.rows, heads, n, p, nv.stream_ptr()))
+
+
+def latent_prep(dkv, w_norm, eps: float, cache, q, q_plain, q_abs, inv_freq, step, heads: int, d: int, r: int,
+                rank: int, rot: int, interleaved: bool):
+    """cache [pages, page, rank + r] in the activation type; q [T, heads*(d+r)] fp32; q_plain [T, heads*d] in the
+    activation type; q_abs [T, heads*(rank+r)] fp32 (its rotated columns are written here)."""
+    tokens = q.shape[0]
+    assert dkv.shape == (tokens, rank + r) and w_norm.numel() == rank and w_norm.is_contiguous()
+    assert cache.is_contiguous() and cache.shape[1:] == (step.page, rank + r) and int(step.max_page) < cache.shape[0]
+    assert q.shape == (tokens, heads * (d + r)) and q_plain.shape == (tokens, heads * d)
+    assert q_abs.shape == (tokens, heads * (rank + r)) and q_plain.dtype == cache.dtype and step.tokens == tokens
+    assert rot == 0 or (inv_freq.is_cuda and inv_freq.dtype == torch.float64 and inv_freq.numel() == rot // 2)
+    nv.check("mv_latent_prep", nv.lib().mv_latent_prep(
+        _f32(dkv).data_ptr(), _ld(dkv), _f32(w_norm).data_ptr(), float(eps), cache.data_ptr(), _f32(q).data_ptr(),
+        _ld(q), q_plain.data_ptr(), _ld(q_plain), _f32(q_abs).data_ptr(), _ld(q_abs),
+        None if rot == 0 else inv_freq.data_ptr(), step.tok_row.data_ptr(), step.tok_pos.data_ptr(),
+        step.block_table.data_ptr(), step.block_table.stride(0), step.page, tokens, heads, d, r, rank, rot,
+        int(interleaved), _is_f32(cache), nv.stream_ptr()))
+
+
+def latent_attn(q_abs, cache, out, step, sinks, heads: int, rank: int, r: int, scale: float, window: int):
+    """out [T, heads*rank] in the activation type: weighted sums of the cached latents.  window 0: causal."""
+    tokens = q_abs.shape[0]
+    assert q_abs.shape == (tokens, heads * (rank + r)) and out.shape == (tokens, heads * rank)
+    assert cache.is_contiguous() and cache.shape[1:] == (step.page, rank + r) and int(step.max_page) < cache.shape[0]
+    assert out.dtype == cache.dtype and step.tokens == tokens
+    assert sinks is None or (sinks.numel() == heads and sinks.is_contiguous())
+    nv.check("mv_latent_attn", nv.lib().mv_latent_attn(
+        _f32(q_abs).data_ptr(), _ld(q_abs), cache.data_ptr(), out.data_ptr(), _ld(out), step.tok_row.data_ptr(),
+        step.tok_pos.data_ptr(), step.block_table.data_ptr(), step.block_table.stride(0), step.page,
+        None if sinks is None else _f32(sinks).data_ptr(), tokens, heads, rank, r, float(scale), int(window),
+        _is_f32(cache), nv.stream_ptr()))
+
+
+def moe_route(h, w_router, w_shared_gate, ids, weights, shared_gate):
+    tokens, n = h.shape
+    E, top = w_router.shape[0], ids.shape[1]
+    assert h.stride(1) == 1 and w_router.shape == (E, n) and w_router.is_contiguous()
+    assert ids.shape == (tokens, top) and weights.shape == (tokens, top) and ids.is_contiguous()
+    assert weights.is_contiguous() and ids.dtype == torch.int32
+    assert w_shared_gate is None or (w_shared_gate.numel() == n and w_shared_gate.is_contiguous()
+                                     and shared_gate.numel() == tokens and shared_gate.is_contiguous())
+    nv.check("mv_moe_route", nv.lib().mv_moe_route(
+        h.data_ptr(), _ld(h), _f32(w_router).data_ptr(), None if w_shared_gate is None else _f32(w_shared_gate).data_ptr(),
+        ids.data_ptr(), _f32(weights).data_ptr(), None if w_shared_gate is None else _f32(shared_gate).data_ptr(),
+        tokens, n, E, top, _is_f32(h), nv.stream_ptr()))
+
+
+def moe_plan(ids, seg, order, place, experts: int):
+    pairs = ids.numel()
+    assert seg.numel() == experts + 1 and order.numel() == pairs and place.numel() == pairs
+    nv.check("mv_moe_plan", nv.lib().mv_moe_plan(
+        _i32(ids).data_ptr(), _i32(seg).data_ptr(), _i32(order).data_ptr(), _i32(place).data_ptr(), pairs, experts,
+        nv.stream_ptr()))
+
+
+def moe_combine(expert_out, place, weights, shared_out, shared_gate, y):
+    tokens, n = y.shape
+    top = weights.shape[1]
+    assert expert_out.shape == (tokens * top, n) and place.numel() == tokens * top and weights.is_contiguous()
+    assert shared_out is None or (shared_out.shape == (tokens, n) and shared_gate.numel() == tokens)
+    nv.check("mv_moe_combine", nv.lib().mv_moe_combine(
+        _f32(expert_out).data_ptr(), _ld(expert_out), _i32(place).data_ptr(), _f32(weights).data_ptr(),
+        None if shared_out is None else _f32(shared_out).data_ptr(), 0 if shared_out is None else _ld(shared_out),
+        None if shared_out is None else _f32(shared_gate).data_ptr(), _f32(y).data_ptr(), _ld(y), tokens, n, top,
+        nv.stream_ptr()))

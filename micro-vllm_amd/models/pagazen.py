@@ -49,6 +49,10 @@ class PagazenConfig:
         j = self.layers[i].get("weights_of", i)
         return i if j is None else int(j)
 
+    def layer_runs(self):
+        """[(index of the layer whose tensors the run uses, its description)] in running order."""
+        return [(self.weights_layer(i), layer) for i, layer in enumerate(self.layers)]
+
     @classmethod
     def from_json(cls, d: dict, name: str = "pagazen") -> "PagazenConfig":
         layers = d["layers"]

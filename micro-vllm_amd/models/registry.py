@@ -5,8 +5,8 @@ A family = (configuration reader, model object, runner and cache manager the eng
              graph-captured single-token decode over one KV geometry (ModelPrefillRunner /
              ModelGraphRunner / KVCacheManager);
   "ragged" - stacks with an fp32 residual stream whose layers are listed one by one (recurrent
-             mixers, windowed attention), run step by step over ragged batches (RaggedRunner /
-             HybridCacheManager).
+             mixers, windowed or latent attention, dense or routed feed-forwards), run step by step
+             over ragged batches (RaggedRunner / HybridCacheManager): Pagazen, Fagunex.
 """
 from typing import Callable, Dict
 
@@ -27,7 +27,17 @@ def _load_pagazen(config_json, files, name):
     return PagazenModel(cfg, files)
 
 
+def _load_fagunex(config_json, files, name):
+    from .fagunex import FagunexConfig, FagunexModel, tensor_shapes
+    cfg = FagunexConfig.from_json(config_json, name)
+    for tensor, shape in tensor_shapes(cfg).items():
+        if tensor not in files:
+            raise KeyError(f"tensor {tensor!r} {shape} is not in the checkpoint")
+    return FagunexModel(cfg, files)
+
+
 register("Pagazen", _load_pagazen)
+register("Fagunex", _load_fagunex)
 
 
 def loader_for(config_json: dict):
