@@ -72,6 +72,13 @@ def parse():
                          "one JSON line of its own")
     ap.add_argument("--pagazen-widths", default="1024,2048,4096")
     ap.add_argument("--pagazen-kernels", action="store_true", help="with --pagazen: per-op times of one layer pair on stderr")
+    ap.add_argument("--fagunex", action="store_true",
+                    help="instead of the default workload: prefill and decode throughput of the Fagunex design "
+                         "(Dynamic Tanh norms, gated recurrence, attention over a cached latent, routed experts; "
+                         "random weights) at a few widths, beside Pagazen - the other design of the ragged family - "
+                         "at equal width and depth; one JSON line of its own")
+    ap.add_argument("--fagunex-widths", default="1024,2048,4096")
+    ap.add_argument("--fagunex-kernels", action="store_true", help="with --fagunex: per-op times of one step on stderr")
     return ap.parse_args()
 
 
@@ -625,6 +632,55 @@ def pagazen_compare(args, dev):
                       "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "n_gpus": 1, "rows": rows}), flush=True)
 
 
+def _ragged_engine_row(eng, cfg, S, prefix, kernels, width):
+    """Prefill of one prompt of S tokens and decode at bs 1 / 8 behind it, through InferenceEngine.run_ragged."""
+    row = {}
+    ids = torch.randint(0, cfg.vocab_size, (S,), generator=torch.Generator().manual_seed(0)).tolist()
+
+    def prefill():
+        eng.run_ragged([("p", ids, [S - 1])])
+        eng.release("p")
+    ms = _events_ms(prefill, 3)
+    row[f"{prefix}_prefill_tok_s"] = round(S / ms * 1e3, 1)
+    for bs in (1, 8):
+        for i in range(bs):
+            eng.run_ragged([(i, ids, [])])
+        ms = _events_ms(lambda: eng.run_ragged([(i, [7], [0]) for i in range(bs)]), 20)
+        row[f"{prefix}_decode_bs{bs}_tok_s"] = round(bs / ms * 1e3, 1)
+        row[f"{prefix}_decode_bs{bs}_ms"] = round(ms, 3)
+        for i in range(bs):
+            eng.release(i)
+    row[f"{prefix}_weight_GB"] = round(eng.runner.weight_bytes / 1e9, 3)
+    if kernels:
+        pagazen_kernel_table(eng, ids, f"{prefix} {width}")
+    return row
+
+
+def fagunex_compare(args, dev):
+    """Prefill (one prompt of --ctx tokens) and decode (bs 1 and 8 at context --ctx) of the Fagunex design beside
+    Pagazen at equal width and depth, both through InferenceEngine.run_ragged.  Random weights, 4 layers per
+    model (3 recurrent + 1 attention each), vocabulary 32000.  Fagunex: 8 experts of which 2 are used plus a
+    shared one, together 4 x width of active feed-forward; Pagazen: a dense feed-forward of 4 x width."""
+    import micro_vllm_amd  # noqa: F401
+    from micro_vllm_amd.core.engine import InferenceEngine
+    from micro_vllm_amd.models import fagunex, pagazen
+
+    S, layers, rows = args.ctx, 4, []
+    for width in [int(w) for w in args.fagunex_widths.split(",")]:
+        row = {"width": width, "layers": layers, "ctx": S}
+        for name, mod in (("fagunex", fagunex), ("pagazen", pagazen)):
+            cfg = mod.bench_config(width, layers)
+            eng = InferenceEngine(model=mod.build_random_model(cfg, seed=1), max_batch_size=8, max_prefill_tokens=S,
+                                  n_blocks=9 * (S // 64 + 4), max_tokens=S + 256, state_slots=9)
+            row.update(_ragged_engine_row(eng, cfg, S, name, args.fagunex_kernels, width))
+            del eng
+            torch.cuda.empty_cache()
+        log(f"[bench] {row}")
+        rows.append(row)
+    print(json.dumps({"metric": "Fagunex beside Pagazen (ragged family): prefill and decode tokens/s at equal size",
+                      "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "n_gpus": 1, "rows": rows}), flush=True)
+
+
 def pagazen_kernel_table(eng, ids, width):
     """Per-op time of one prefill step and one single-token step (rocprof-free: HIP events around each
     wrapper call), printed on stderr."""
@@ -632,7 +688,10 @@ def pagazen_kernel_table(eng, ids, width):
     import functools
     times = {}
     names = ["embed_scaled", "postnorm_residual", "offset_rmsnorm_gather", "relu_squared", "softcap_", "conv_silu",
-             "softplus_decay", "scan_outer", "rotary_pairs_", "gated_group_norm", "qk_unitnorm_store", "window_attn"]
+             "softplus_decay", "scan_outer", "rotary_pairs_", "gated_group_norm", "qk_unitnorm_store", "window_attn",
+             "dyt_shift", "dyt_gather", "dyt_residual", "unitnorm_residual", "rmsnorm_rows", "gelu_gate_rows", "silu_mul",
+             "sigmoid_gate", "linear_heads", "linear_segments", "gate_lower_bound_", "scan_gated", "latent_prep",
+             "latent_attn", "moe_route", "moe_plan", "moe_combine"]
     saved = {n: getattr(ops, n) for n in names}
     saved_call = ops.AnyLinear.__call__
 
@@ -761,6 +820,9 @@ def main():
     if args.pagazen:
         assert world == 1, "--pagazen runs on one GPU"
         return pagazen_compare(args, dev)
+    if args.fagunex:
+        assert world == 1, "--fagunex runs on one GPU"
+        return fagunex_compare(args, dev)
     peers = world > 1                 # ranks to synchronise with
     if args.as_rank_of:
         assert world == 1, "--as-rank-of runs one process"

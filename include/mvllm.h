@@ -609,10 +609,15 @@ int mv_linear_segments(const void* x, int64_t ldx, const void* w, int64_t ldw, i
 int mv_gate_lower_bound(float* q, int64_t ldq, float* f, int64_t ldf, const float* bias, const float* lower,
                         int tokens, int n, mv_stream_t stream);
 /* S_t = diag(f_t) S_(t-1) + (1 - f_t) v_t^T, o_t = S_t^T q_t per head; q, f [T, heads*n], v, out [T, heads*p],
- * state [slots, heads, n, p] fp32 (taken as zero when row_ctx == 0). */
+ * state [slots, heads, n, p] fp32 (taken as zero when row_ctx == 0).  chunks > 0: rows longer than max_len are cut
+ * into chunks (ch_start / ch_len / row_ch0 / row_nch as for mv_scan_chunked) that run side by side from a zero
+ * state and are then joined through the products of their gates (scratch: ds [chunks, heads, n, p], cum
+ * [tokens, heads*n], fp32); differs from the token-by-token form by the order of the fp32 sums only. */
 int mv_scan_gated(const float* q, int64_t ldq, const float* f, int64_t ldf, const float* v, int64_t ldv, float* state,
                   float* out, int64_t ldo, const int32_t* row_start, const int32_t* row_len, const int32_t* row_ctx,
-                  const int32_t* row_slot, int rows, int heads, int n, int p, mv_stream_t stream);
+                  const int32_t* row_slot, int rows, int heads, int n, int p, float* ds, float* cum,
+                  const int32_t* ch_start, const int32_t* ch_len, const int32_t* row_ch0, const int32_t* row_nch,
+                  int chunks, int max_len, mv_stream_t stream);
 
 /* ---- attention over a cached latent (latent_attn.hip) ------------------------------------------------ */
 

@@ -120,7 +120,8 @@ PROTOTYPES = {
     "mv_linear_heads": (_I, [_P, _L, _L, _P, _L, _L, _P, _L, _L, _I, _I, _I, _I, _I, _P]),
     "mv_linear_segments": (_I, [_P, _L, _P, _L, _L, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
     "mv_gate_lower_bound": (_I, [_P, _L, _P, _L, _P, _P, _I, _I, _P]),
-    "mv_scan_gated": (_I, [_P, _L, _P, _L, _P, _L, _P, _P, _L, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "mv_scan_gated": (_I, [_P, _L, _P, _L, _P, _L, _P, _P, _L, _P, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P,
+                           _I, _I, _P]),
     "mv_latent_prep": (_I, [_P, _L, _P, _F, _P, _P, _L, _P, _L, _P, _L, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I,
                             _I, _I, _I, _P]),
     "mv_latent_attn": (_I, [_P, _L, _P, _P, _L, _P, _P, _P, _I, _I, _P, _I, _I, _I, _I, _F, _I, _I, _P]),

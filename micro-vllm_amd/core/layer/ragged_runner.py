@@ -400,7 +400,7 @@ class RaggedRunner:
         q, f, v = proj[:, :H * n], proj[:, H * n:2 * H * n], proj[:, 2 * H * n:]
         ops.gate_lower_bound_(q, f, w["f_b"], w["lower"])
         o = self._f32buf(T, H * p)
-        ops.scan_gated(q, f, v, cache.states[li]["gated"], o, step, H, n, p)
+        ops.scan_gated(q, f, v, cache.states[li]["gated"], o, step, H, n, p, chunked=self.chunked_scan)
         u = self._actbuf(T, H * p)
         ops.rmsnorm_rows(o, w["norm"], self.cfg.eps, u, per=H)
         return w["w_o"](u, self._f32buf(T, self.width))

@@ -107,6 +107,10 @@ struct ScanArgs {
     StepRows r;
     int H, n, p, pt;
     int max_len;   // rows longer than this belong to the chunked form (0: every row is taken)
+    // chunk mode (ch_start != NULL): blockIdx.z is a chunk of a long row, run from a zero state; what it
+    // leaves goes to ds[chunk][head] instead of the slot
+    const int *ch_start, *ch_len;
+    float* ds;
 };
 
 // GATED: `decay` holds a forget gate per (token, head, state row) and the key is one minus it.
@@ -118,10 +122,12 @@ __global__ __launch_bounds__(256) void scan_outer_kernel(ScanArgs a) {
     const int cl = tid % PT, ng = tid / PT, c = blockIdx.x * PT + cl;
     const bool vc = c < a.p;
     const int npt = (a.n + NS - 1) / NS, n0 = ng * npt;
-    const int len = a.r.row_len[b], start = a.r.row_start[b];
-    if (a.max_len > 0 && len > a.max_len) return;   // the whole workgroup
-    const bool carried = a.r.row_ctx[b] > 0;
-    float* sp = a.state + (((int64_t)a.r.row_slot[b] * a.H + h) * a.n + n0) * a.p + c;
+    const bool chunk = a.ch_start != nullptr;
+    const int len = chunk ? a.ch_len[b] : a.r.row_len[b], start = chunk ? a.ch_start[b] : a.r.row_start[b];
+    if (!chunk && a.max_len > 0 && len > a.max_len) return;   // the whole workgroup
+    const bool carried = !chunk && a.r.row_ctx[b] > 0;
+    float* sp = (chunk ? a.ds + (((int64_t)b * a.H + h) * a.n + n0) * a.p
+                       : a.state + (((int64_t)a.r.row_slot[b] * a.H + h) * a.n + n0) * a.p) + c;
     float S[MAXN];
 #pragma unroll
     for (int i = 0; i < MAXN; ++i) S[i] = (carried && vc && i < npt && n0 + i < a.n) ? sp[(int64_t)i * a.p] : 0.f;
@@ -392,6 +398,110 @@ __global__ __launch_bounds__(256) void scan_chunk_inter_kernel(ChunkArgs a) {
                         *op = res;
                     }
             }
+        }
+    }
+}
+
+// ---- the gated recurrence in chunks of 64 tokens ----
+// Within a chunk that starts from state S0, with P_t[i] the product of the gates f_s[i] over the chunk's tokens
+// s <= t:  o_t = (local run from a zero state)_t + sum_i q_t[i] P_t[i] S0[i][:],  S_end = diag(P_end) S0 + local.
+//   gate_cumprod   P_t for every token of every chunk
+//   scan_outer_kernel in chunk mode: the local runs, all chunks side by side
+//   gated_carry    per (row, head): the state each chunk starts from, in turn (left where the local sum was),
+//                  and the row's final state
+//   gated_inter    o_t += (q_t * P_t) S0, a [64 x n] . [n x p] product per (chunk, head) in fp32
+// Products of gates, no logarithms: a gate of exactly zero or one is exact, long decays underflow to zero as
+// the token-by-token run does.
+__global__ __launch_bounds__(256) void gate_cumprod_kernel(const float* f, int64_t ldf, float* cum, int64_t ldc,
+                                                           const int* ch_start, const int* ch_len, int width) {
+    const int ch = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= width) return;
+    const int start = ch_start[ch], len = ch_len[ch];
+    float pr = 1.0f;
+    for (int t = 0; t < len; ++t) {
+        pr *= f[(int64_t)(start + t) * ldf + c];
+        cum[(int64_t)(start + t) * ldc + c] = pr;
+    }
+}
+
+struct GatedChunkArgs {
+    const float* q;
+    const float* cum;
+    int64_t ldq, ldc, ldo;
+    float* state;
+    float* out;
+    float* ds;
+    const int *ch_start, *ch_len, *row_ch0, *row_nch, *row_ctx, *row_slot;
+    int H, n, p;
+};
+
+__global__ __launch_bounds__(256) void gated_carry_kernel(GatedChunkArgs a) {
+    const int b = blockIdx.z, h = blockIdx.y;
+    const int np = a.n * a.p, e = blockIdx.x * 256 + threadIdx.x;
+    const int nch = a.row_nch[b];
+    if (nch == 0 || e >= np) return;
+    const int i = e / a.p;
+    float* sp = a.state + ((int64_t)a.row_slot[b] * a.H + h) * np + e;
+    float S = a.row_ctx[b] > 0 ? *sp : 0.f;
+    const int c0 = a.row_ch0[b];
+    for (int c = c0; c < c0 + nch; ++c) {
+        float* d = a.ds + ((int64_t)c * a.H + h) * np + e;
+        const float add = *d;
+        *d = S;                                   // the state this chunk starts from
+        const int last = a.ch_start[c] + a.ch_len[c] - 1;
+        S = fmaf(a.cum[(int64_t)last * a.ldc + (int64_t)h * a.n + i], S, add);
+    }
+    *sp = S;
+}
+
+// one workgroup per (chunk, head, 64 value columns): thread (ty, tx) owns 4 tokens x 4 columns
+__global__ __launch_bounds__(256) void gated_inter_kernel(GatedChunkArgs a) {
+    __shared__ float as[16][kCh + 4];
+    __shared__ float ss[16][64 + 4];
+    const int ch = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * 64;
+    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    const int start = a.ch_start[ch], len = a.ch_len[ch];
+    const float* S0 = a.ds + ((int64_t)ch * a.H + h) * a.n * a.p;
+    const int lrow = tid >> 2, lcol = (tid & 3) * 4;
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < a.n; k0 += 16) {
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int kk = k0 + lcol + i;
+            const bool ok = lrow < len && kk < a.n;
+            const int64_t tok = start + lrow;
+            as[lcol + i][lrow] = ok ? a.q[tok * a.ldq + (int64_t)h * a.n + kk] * a.cum[tok * a.ldc + (int64_t)h * a.n + kk] : 0.f;
+        }
+        {   // the state tile: thread (k = tid / 16, four neighbouring columns)
+            const int sk = k0 + (tid >> 4), sc = c0 + (tid & 15) * 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                ss[tid >> 4][(tid & 15) * 4 + i] = (sk < a.n && sc + i < a.p) ? S0[(int64_t)sk * a.p + sc + i] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk) {
+            float x[4], y[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                x[i] = as[kk][ty * 4 + i];
+                y[i] = ss[kk][tx * 4 + i];
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(x[i], y[j], acc[i][j]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int t = ty * 4 + i;
+        if (t >= len) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = c0 + tx * 4 + j;
+            if (c < a.p) a.out[(int64_t)(start + t) * a.ldo + (int64_t)h * a.p + c] += acc[i][j];
         }
     }
 }
@@ -823,6 +933,7 @@ int mv_scan_outer(const float* q, int64_t ldq, int q_div, const float* k, int64_
     a.q_div = q_div; a.k_div = k_div; a.state = state; a.out = out;
     a.r = StepRows{nullptr, nullptr, row_start, row_len, row_ctx, row_slot};
     a.H = heads; a.n = n; a.p = p; a.max_len = max_len;
+    a.ch_start = nullptr; a.ch_len = nullptr; a.ds = nullptr;
     a.pt = p % 64 == 0 ? 64 : (p % 32 == 0 ? 32 : 16);
     // a state too tall for 64 rows a thread: narrower column tiles leave more threads to share its rows
     while (a.pt > 16 && (n + 256 / a.pt - 1) / (256 / a.pt) > 64) a.pt /= 2;
@@ -838,28 +949,51 @@ int mv_scan_outer(const float* q, int64_t ldq, int q_div, const float* k, int64_
 
 int mv_scan_gated(const float* q, int64_t ldq, const float* f, int64_t ldf, const float* v, int64_t ldv, float* state,
                   float* out, int64_t ldo, const int32_t* row_start, const int32_t* row_len, const int32_t* row_ctx,
-                  const int32_t* row_slot, int rows, int heads, int n, int p, mv_stream_t stream) {
+                  const int32_t* row_slot, int rows, int heads, int n, int p, float* ds, float* cum,
+                  const int32_t* ch_start, const int32_t* ch_len, const int32_t* row_ch0, const int32_t* row_nch,
+                  int chunks, int max_len, mv_stream_t stream) {
     using namespace mv;
-    if (rows < 0 || heads <= 0 || n <= 0 || p <= 0) return MV_ERR_INVALID_ARG;
+    if (rows < 0 || heads <= 0 || n <= 0 || p <= 0 || chunks < 0) return MV_ERR_INVALID_ARG;
     if (rows == 0) return MV_OK;
-    if (!q || !f || !v || !state || !out || rows > 65535 || heads > 65535) return MV_ERR_INVALID_ARG;
+    if (!q || !f || !v || !state || !out || rows > 65535 || heads > 65535 || chunks > 65535) return MV_ERR_INVALID_ARG;
     if (ldq < (int64_t)heads * n || ldf < (int64_t)heads * n || ldv < (int64_t)heads * p || ldo < (int64_t)heads * p)
+        return MV_ERR_INVALID_ARG;
+    if (chunks > 0 && (!ds || !cum || !ch_start || !ch_len || !row_ch0 || !row_nch || max_len <= 0))
         return MV_ERR_INVALID_ARG;
     ScanArgs a;
     a.q = q; a.k = nullptr; a.v = v; a.decay = f; a.gain = nullptr; a.skip = nullptr;
     a.ldq = ldq; a.ldk = 0; a.ldv = ldv; a.ld_decay = ldf; a.ld_gain = 0; a.ldo = ldo;
     a.q_div = 1; a.k_div = 1; a.state = state; a.out = out;
     a.r = StepRows{nullptr, nullptr, row_start, row_len, row_ctx, row_slot};
-    a.H = heads; a.n = n; a.p = p; a.max_len = 0;
+    a.H = heads; a.n = n; a.p = p; a.max_len = chunks > 0 ? max_len : 0;
+    a.ch_start = nullptr; a.ch_len = nullptr; a.ds = nullptr;
     a.pt = p % 64 == 0 ? 64 : (p % 32 == 0 ? 32 : 16);
     while (a.pt > 16 && (n + 256 / a.pt - 1) / (256 / a.pt) > 64) a.pt /= 2;
     const int ns = 256 / a.pt, npt = (n + ns - 1) / ns;
-    const dim3 grid((p + a.pt - 1) / a.pt, heads, rows);
+    if (npt > 64) return MV_ERR_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
-    if (npt <= 4) hipLaunchKernelGGL((scan_outer_kernel<4, true>), grid, dim3(256), 0, s, a);
-    else if (npt <= 16) hipLaunchKernelGGL((scan_outer_kernel<16, true>), grid, dim3(256), 0, s, a);
-    else if (npt <= 64) hipLaunchKernelGGL((scan_outer_kernel<64, true>), grid, dim3(256), 0, s, a);
-    else return MV_ERR_UNSUPPORTED;
+    const int tiles = (p + a.pt - 1) / a.pt;
+    // rows of up to max_len tokens (all rows when nothing is cut into chunks): token by token from the slot's state
+    for (int pass = 0; pass < (chunks > 0 ? 2 : 1); ++pass) {
+        if (pass == 1) {
+            a.ch_start = ch_start; a.ch_len = ch_len; a.ds = ds;
+        }
+        const dim3 grid(tiles, heads, pass == 0 ? rows : chunks);
+        if (npt <= 4) hipLaunchKernelGGL((scan_outer_kernel<4, true>), grid, dim3(256), 0, s, a);
+        else if (npt <= 16) hipLaunchKernelGGL((scan_outer_kernel<16, true>), grid, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL((scan_outer_kernel<64, true>), grid, dim3(256), 0, s, a);
+    }
+    if (chunks > 0) {
+        const int width = heads * n;
+        hipLaunchKernelGGL(gate_cumprod_kernel, dim3(chunks, (width + 255) / 256), dim3(256), 0, s, f, ldf, cum,
+                           (int64_t)width, ch_start, ch_len, width);
+        GatedChunkArgs g;
+        g.q = q; g.cum = cum; g.ldq = ldq; g.ldc = width; g.ldo = ldo; g.state = state; g.out = out; g.ds = ds;
+        g.ch_start = ch_start; g.ch_len = ch_len; g.row_ch0 = row_ch0; g.row_nch = row_nch; g.row_ctx = row_ctx;
+        g.row_slot = row_slot; g.H = heads; g.n = n; g.p = p;
+        hipLaunchKernelGGL(gated_carry_kernel, dim3((n * p + 255) / 256, heads, rows), dim3(256), 0, s, g);
+        hipLaunchKernelGGL(gated_inter_kernel, dim3(chunks, heads, (p + 63) / 64), dim3(256), 0, s, g);
+    }
     return check_launch();
 }
 

@@ -368,17 +368,26 @@ def gate_lower_bound_(q, f, bias, lower):
         _f32(lower).data_ptr(), tokens, n, nv.stream_ptr()))
 
 
-def scan_gated(q, f, v, state, out, step, heads: int, n: int, p: int):
-    """S_t = diag(f_t) S_(t-1) + (1 - f_t) v_t^T, o_t = S_t^T q_t; state [slots, heads, n, p] fp32."""
+def scan_gated(q, f, v, state, out, step, heads: int, n: int, p: int, chunked: bool = True):
+    """S_t = diag(f_t) S_(t-1) + (1 - f_t) v_t^T, o_t = S_t^T q_t; state [slots, heads, n, p] fp32.  Rows of up to
+    SCAN_SEQ_MAX tokens run token by token; longer rows in chunks of 64 side by side unless `chunked` is False."""
     tokens = v.shape[0]
     assert q.shape == (tokens, heads * n) and f.shape == (tokens, heads * n)
     assert v.shape == (tokens, heads * p) and out.shape == (tokens, heads * p)
     assert state.is_contiguous() and state.shape[1:] == (heads, n, p) and int(step.max_slot) < state.shape[0]
     assert step.tokens == tokens
+    chunks = step.n_chunks if chunked else 0
+    ds = cum = None
+    if chunks:
+        ds = torch.empty(chunks, heads, n, p, dtype=torch.float32, device=v.device)
+        cum = torch.empty(tokens, heads * n, dtype=torch.float32, device=v.device)
     nv.check("mv_scan_gated", nv.lib().mv_scan_gated(
         _f32(q).data_ptr(), _ld(q), _f32(f).data_ptr(), _ld(f), _f32(v).data_ptr(), _ld(v), _f32(state).data_ptr(),
         _f32(out).data_ptr(), _ld(out), step.row_start.data_ptr(), step.row_len.data_ptr(), step.row_ctx.data_ptr(),
-        step.row_slot.data_ptr(), step.rows, heads, n, p, nv.stream_ptr()))
+        step.row_slot.data_ptr(), step.rows, heads, n, p, None if ds is None else ds.data_ptr(),
+        None if cum is None else cum.data_ptr(), step.ch_start.data_ptr() if chunks else None,
+        step.ch_len.data_ptr() if chunks else None, step.row_ch0.data_ptr() if chunks else None,
+        step.row_nch.data_ptr() if chunks else None, chunks, SCAN_SEQ_MAX, nv.stream_ptr()))
 
 
 def latent_prep(dkv, w_norm, eps: float, cache, q, q_plain, q_abs, inv_freq, step, heads: int, d: int, r: int,

@@ -191,7 +191,7 @@ def bench_config(width: int, n_layers: int, vocab: int = 32000, ff_mult: int = 4
     (alternately the windowed and the causal kind), the others hgrn2; routed experts whose active
     feed-forward width (top experts + the shared one) is ff_mult * width."""
     layers = []
-    ff = ff_mult * width // (top + 1)
+    ff = (ff_mult * width // (top + 1) + 63) // 64 * 64
     mlp = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}, "shared": {"ff": ff}}
     k = 0
     for i in range(n_layers):

@@ -199,6 +199,43 @@ def test_gated_recurrence_over_steps(ops, heads, n, p):
         assert (torch.cat(got[k]).view(lens[k], heads, p) - want[k]).abs().max().item() < 2e-5, k
 
 
+@pytest.mark.parametrize("heads,n,p", [(2, 32, 32), (3, 40, 24), (1, 128, 128), (2, 8, 100)])
+def test_gated_recurrence_in_chunks_against_token_by_token(ops, heads, n, p):
+    """Long rows are cut into chunks of 64 that run side by side and are joined through the products of their
+    gates: against the restatement and against the token-by-token kernel, with gates of exactly zero and one,
+    chunks cut at odd places, a second portion that continues from the slot's state, a short row beside them."""
+    g = torch.Generator().manual_seed(heads + n + p)
+    cache = make_cache(state={0: {"gated": (heads, n, p)}, 1: {"gated": (heads, n, p)}}, max_tokens=1024)
+    for st_ in cache.states.values():
+        st_["gated"].fill_(-2.0)
+    lens = {"a": 450, "b": 9, "c": 131}
+    q = {k: torch.randn(L, heads * n, generator=g) for k, L in lens.items()}
+    f = {k: torch.rand(L, heads * n, generator=g) ** 0.25 for k, L in lens.items()}
+    v = {k: torch.randn(L, heads * p, generator=g) for k, L in lens.items()}
+    f["a"][:, 0], f["a"][:, 1] = 1.0, 0.0
+    f["a"][100:170, 2] = 0.05                       # a product over a chunk that underflows
+    want = {k: ref.gated_write_recurrence(q[k].double().view(-1, heads, n), f[k].double().view(-1, heads, n),
+                                          v[k].double().view(-1, heads, p))[0] for k in lens}
+    got = {True: {k: [] for k in lens}, False: {k: [] for k in lens}}
+    at = {k: 0 for k in lens}
+    for rows in [[("a", 203), ("b", 9), ("c", 17)], [("c", 114), ("a", 247)]]:
+        st = step_of(cache, [(k, [0] * c) for k, c in rows])
+        qs, fs, vs = (torch.cat([x[k][at[k]:at[k] + c] for k, c in rows]).to(DEV) for x in (q, f, v))
+        for li, chunked in ((0, True), (1, False)):
+            out = torch.empty(qs.shape[0], heads * p, device=DEV)
+            ops.scan_gated(qs, fs, vs, cache.states[li]["gated"], out, st, heads, n, p, chunked=chunked)
+            o = 0
+            for k, c in rows:
+                got[chunked][k].append(out[o:o + c].cpu().double())
+                o += c
+        for k, c in rows:
+            at[k] += c
+    for k in lens:
+        a, b = torch.cat(got[True][k]).view(-1, heads, p), torch.cat(got[False][k]).view(-1, heads, p)
+        assert (b - want[k]).abs().max().item() < 2e-5 and (a - want[k]).abs().max().item() < 2e-5, k
+    assert (cache.states[0]["gated"] - cache.states[1]["gated"]).abs().max().item() < 2e-5
+
+
 def latent_case(g, T, H, d, r, dv, R, rot, base):
     q = torch.randn(T, H * (d + r), generator=g)
     dkv = torch.randn(T, R + r, generator=g)
