@@ -598,10 +598,10 @@ int mv_sigmoid_gate(const float* a, int64_t lda, const float* g, int64_t ldg, vo
 int mv_linear_heads(const void* x, int64_t ldx, int64_t zx, const void* w, int64_t ldw, int64_t zw, float* y,
                     int64_t ldy, int64_t zy, int m, int n, int k, int heads, int f32, mv_stream_t stream);
 /* Output rows seg[e] .. seg[e+1] use weight w + e*zw; operand row of output row i is src[i] / src_div (src == NULL:
- * i).  max_rows bounds the rows of one segment. */
+ * i).  max_rows bounds the rows of one segment, total_rows = seg[segments] (the rows of y). */
 int mv_linear_segments(const void* x, int64_t ldx, const void* w, int64_t ldw, int64_t zw, float* y, int64_t ldy,
-                       const int32_t* seg, const int32_t* src, int src_div, int segments, int max_rows, int n, int k,
-                       int f32, mv_stream_t stream);
+                       const int32_t* seg, const int32_t* src, int src_div, int segments, int max_rows, int total_rows,
+                       int n, int k, int f32, mv_stream_t stream);
 
 /* ---- gated recurrence without a key (seq_mix.hip) ---------------------------------------------------- */
 

@@ -118,7 +118,7 @@ PROTOTYPES = {
     "mv_silu_mul": (_I, [_P, _L, _P, _L, _I, _I, _I, _P]),
     "mv_sigmoid_gate": (_I, [_P, _L, _P, _L, _P, _L, _I, _I, _I, _P]),
     "mv_linear_heads": (_I, [_P, _L, _L, _P, _L, _L, _P, _L, _L, _I, _I, _I, _I, _I, _P]),
-    "mv_linear_segments": (_I, [_P, _L, _P, _L, _L, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
+    "mv_linear_segments": (_I, [_P, _L, _P, _L, _L, _P, _L, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
     "mv_gate_lower_bound": (_I, [_P, _L, _P, _L, _P, _P, _I, _I, _P]),
     "mv_scan_gated": (_I, [_P, _L, _P, _L, _P, _L, _P, _P, _L, _P, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P,
                            _I, _I, _P]),

@@ -323,10 +323,14 @@ int mv_latent_attn(const float* q_abs, int64_t ldq, const void* cache, void* out
     hipStream_t s = (hipStream_t)stream;
     // few tokens (decoding): sixteen waves share a token's keys, so that the launch still fills the chip
     const bool few = (int64_t)tokens * ((heads + 3) / 4) < 2 * (int64_t)num_cus();
+    // very few (a handful of decoded tokens): a workgroup per head rather than per four heads
+    const bool alone = (int64_t)tokens * ((heads + 3) / 4) < 64;
     if (f32) {
+        if (alone) return latent_attn_vc<true, 16, 1>(q_abs, ldq, cache, out, ldo, pr, sinks, tokens, heads, rank, r, scale, window, s);
         if (few) return latent_attn_vc<true, 16, 4>(q_abs, ldq, cache, out, ldo, pr, sinks, tokens, heads, rank, r, scale, window, s);
         return latent_attn_vc<true, 4, 4>(q_abs, ldq, cache, out, ldo, pr, sinks, tokens, heads, rank, r, scale, window, s);
     }
+    if (alone) return latent_attn_vc<false, 16, 1>(q_abs, ldq, cache, out, ldo, pr, sinks, tokens, heads, rank, r, scale, window, s);
     if (few) return latent_attn_vc<false, 16, 4>(q_abs, ldq, cache, out, ldo, pr, sinks, tokens, heads, rank, r, scale, window, s);
     return latent_attn_vc<false, 4, 4>(q_abs, ldq, cache, out, ldo, pr, sinks, tokens, heads, rank, r, scale, window, s);
 }

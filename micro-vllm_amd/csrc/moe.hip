@@ -28,9 +28,11 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const void* h_, int64_t 
         float dot = 0.f;
         if (F32) {
             const float* h = (const float*)h_ + (int64_t)t * ldh;
+#pragma unroll 8
             for (int c = lane; c < n; c += 64) dot = fmaf(h[c], w[c], dot);
         } else {
             const uint16_t* h = (const uint16_t*)h_ + (int64_t)t * ldh;
+#pragma unroll 8
             for (int c = lane; c < n; c += 64) dot = fmaf(bf16_bits_to_f32(h[c]), w[c], dot);
         }
         dot = wave_sum(dot);
@@ -106,7 +108,8 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* eo, int64
         w[k] = wts[(int64_t)t * top + k];
     }
     const float g = so ? shared_gate[t] : 0.f;
-    for (int c = threadIdx.x; c < n; c += 256) {
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c < n) {
         float acc = 0.f;
         for (int k = 0; k < top; ++k) acc = fmaf(w[k], eo[(int64_t)rows[k] * lde + c], acc);
         if (so) acc = fmaf(g, so[(int64_t)t * lds_ + c], acc);
@@ -151,7 +154,7 @@ int mv_moe_combine(const float* expert_out, int64_t lde, const int32_t* place, c
     if (!expert_out || !place || !weights || !y || (shared_out && !shared_gate) || lde < n || ldy < n ||
         (shared_out && lds < n))
         return MV_ERR_INVALID_ARG;
-    hipLaunchKernelGGL(moe_combine_kernel, dim3(tokens), dim3(256), 0, (hipStream_t)stream, expert_out, lde, place,
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(tokens, (n + 255) / 256), dim3(256), 0, (hipStream_t)stream, expert_out, lde, place,
                        weights, shared_out, lds, shared_gate, y, ldy, n, top);
     return check_launch();
 }

@@ -131,7 +131,9 @@ __global__ __launch_bounds__(256) void dyt_shift_kernel(const float* x, int64_t 
     const bool carried = row_ctx[r] > 0;
     const float* prev = x + (int64_t)(t - 1) * ldx;
     const float* last = x + (int64_t)(first + len - 1) * ldx;
-    for (int c = threadIdx.x; c < n; c += 256) {
+    // one value per thread (blockIdx.y walks the row): a row alone in its step is spread over many workgroups
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c < n) {
         const float nc = fmaf(tanhf(al * cur[c]), w[c], b[c]);
         float np;
         if (head) np = carried ? kept[c] : 0.f;
@@ -150,8 +152,8 @@ __global__ __launch_bounds__(256) void dyt_gather_kernel(const float* x, int64_t
     const int row = blockIdx.x;
     const float* a = x + (int64_t)(idx ? idx[row] : row) * ldx;
     const float al = alpha[0];
-    for (int c = threadIdx.x; c < n; c += 256)
-        Act<F32>::st(out + (int64_t)row * ldo + c, fmaf(tanhf(al * a[c]), w[c], b[c]));
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c < n) Act<F32>::st(out + (int64_t)row * ldo + c, fmaf(tanhf(al * a[c]), w[c], b[c]));
 }
 
 template <bool F32>
@@ -162,7 +164,8 @@ __global__ __launch_bounds__(256) void dyt_residual_kernel(const float* y, int64
     T* h = (T*)h_;
     const int row = blockIdx.x;
     const float al = alpha[0];
-    for (int c = threadIdx.x; c < n; c += 256) {
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c < n) {
         const float s = x[(int64_t)row * ldx + c] + fmaf(tanhf(al * y[(int64_t)row * ldy + c]), w[c], b[c]);
         x[(int64_t)row * ldx + c] = s;
         if (h) Act<F32>::st(h + (int64_t)row * ldh + c, s);
@@ -178,9 +181,11 @@ __global__ __launch_bounds__(256) void unitnorm_residual_kernel(const float* y, 
     const int row = blockIdx.x;
     const float* a = y + (int64_t)row * ldy;
     float ss = 0.f;
+#pragma unroll 4
     for (int c = threadIdx.x; c < n; c += 256) ss += a[c] * a[c];
     ss = block_sum(ss, red);
     const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+#pragma unroll 4
     for (int c = threadIdx.x; c < n; c += 256) {
         const float s = x[(int64_t)row * ldx + c] + (a[c] * inv) * w[c];
         x[(int64_t)row * ldx + c] = s;
@@ -200,9 +205,11 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const float* v, int64
     const float* a = v + (r / per) * ld + (r % per) * n;
     T* o = out + (r / per) * ldo + (r % per) * n;
     float ss = 0.f;
+#pragma unroll 4
     for (int c = lane; c < n; c += 64) ss += a[c] * a[c];
     ss = wave_sum(ss);
     const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+#pragma unroll 4
     for (int c = lane; c < n; c += 64) Act<F32>::st(o + c, (a[c] * inv) * w[c]);
 }
 
@@ -221,7 +228,8 @@ __global__ __launch_bounds__(256) void gelu_gate_rows_kernel(const float* a, int
     const int row = blockIdx.x;
     int id = ids[row];
     id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
-    for (int c = threadIdx.x; c < n; c += 256) {
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c < n) {
         const float e = Act<F32>::ld(table + (int64_t)id * ldt + off + c);
         Act<F32>::st(out + (int64_t)row * ldo + c, gelu_tanh_f(a[(int64_t)row * lda + c]) * e);
     }
@@ -331,7 +339,7 @@ int mv_dyt_shift(const float* x, int64_t ldx, const float* w, const float* b, co
         !row_slot || ldx < n || ldh < n)
         return MV_ERR_INVALID_ARG;
     hipStream_t s = (hipStream_t)stream;
-    MV_F32_LAUNCH(dyt_shift_kernel, dim3(tokens), x, ldx, w, b, alpha, mix, state, h, ldh, tok_row, row_start, row_len,
+    MV_F32_LAUNCH(dyt_shift_kernel, dim3(tokens, (n + 255) / 256), x, ldx, w, b, alpha, mix, state, h, ldh, tok_row, row_start, row_len,
                   row_ctx, row_slot, n);
     return check_launch();
 }
@@ -343,7 +351,7 @@ int mv_dyt_gather(const float* x, int64_t ldx, const int32_t* idx, const float* 
     if (rows == 0) return MV_OK;
     if (!x || !w || !b || !alpha || !out || ldx < n || ldo < n) return MV_ERR_INVALID_ARG;
     hipStream_t s = (hipStream_t)stream;
-    MV_F32_LAUNCH(dyt_gather_kernel, dim3(rows), x, ldx, idx, w, b, alpha, out, ldo, n);
+    MV_F32_LAUNCH(dyt_gather_kernel, dim3(rows, (n + 255) / 256), x, ldx, idx, w, b, alpha, out, ldo, n);
     return check_launch();
 }
 
@@ -354,7 +362,7 @@ int mv_dyt_residual(const float* y, int64_t ldy, const float* w, const float* b,
     if (rows == 0) return MV_OK;
     if (!y || !w || !b || !alpha || !x || ldy < n || ldx < n || (h && ldh < n)) return MV_ERR_INVALID_ARG;
     hipStream_t s = (hipStream_t)stream;
-    MV_F32_LAUNCH(dyt_residual_kernel, dim3(rows), y, ldy, w, b, alpha, x, ldx, h, ldh, n);
+    MV_F32_LAUNCH(dyt_residual_kernel, dim3(rows, (n + 255) / 256), y, ldy, w, b, alpha, x, ldx, h, ldh, n);
     return check_launch();
 }
 
@@ -388,7 +396,7 @@ int mv_gelu_gate_rows(const float* a, int64_t lda, const void* table, int64_t ld
     if (rows == 0) return MV_OK;
     if (!a || !table || !ids || !out || lda < n || ldt < off + n || ldo < n) return MV_ERR_INVALID_ARG;
     hipStream_t s = (hipStream_t)stream;
-    MV_F32_LAUNCH(gelu_gate_rows_kernel, dim3(rows), a, lda, table, ldt, off, ids, vocab, out, ldo, n);
+    MV_F32_LAUNCH(gelu_gate_rows_kernel, dim3(rows, (n + 255) / 256), a, lda, table, ldt, off, ids, vocab, out, ldo, n);
     return check_launch();
 }
 

@@ -354,8 +354,8 @@ def linear_segments(x, w, out, seg, src, src_div: int, max_rows: int):
         return out
     nv.check("mv_linear_segments", nv.lib().mv_linear_segments(
         x.data_ptr(), _ld(x), w.data_ptr(), k, n * k, out.data_ptr(), _ld(out), _i32(seg).data_ptr(),
-        None if src is None else _i32(src).data_ptr(), src_div, E, min(max_rows, out.shape[0]), n, k, _is_f32(x),
-        nv.stream_ptr()))
+        None if src is None else _i32(src).data_ptr(), src_div, E, min(max_rows, out.shape[0]), out.shape[0], n, k,
+        _is_f32(x), nv.stream_ptr()))
     return out
 
 

@@ -142,11 +142,23 @@ def test_products_per_head(ops, f32, m, heads, n, k):
     assert bool((wide[:, :, n:] == 9.0).all())
 
 
+@pytest.mark.parametrize("m,n,k", [(300, 130, 96), (513, 256, 40), (260, 128, 64)])
+def test_many_rows_take_the_wide_tile_with_the_same_bits(ops, m, n, k):
+    g = torch.Generator().manual_seed(m)
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16).to(DEV)
+    w = (torch.randn(n, k, generator=g) / math.sqrt(k)).to(torch.bfloat16).to(DEV)
+    lin = ops.AnyLinear(w, wave_tiles=False)
+    got = lin(x)
+    assert (got.cpu().double() - x.cpu().double() @ w.cpu().double().T).abs().max().item() < 1e-4 * math.sqrt(k)
+    for lo in (0, 100, m - 70):           # the same rows in a launch of few rows: the 64 x 64 tile
+        assert torch.equal(lin(x[lo:lo + 70]), got[lo:lo + 70])
+
+
 @pytest.mark.parametrize("f32", [False, True])
-def test_products_by_segment(ops, f32):
+@pytest.mark.parametrize("T,top,E,n,k", [(75, 2, 5, 40, 72), (300, 2, 5, 136, 64), (9, 3, 16, 48, 128)])
+def test_products_by_segment(ops, f32, T, top, E, n, k):
     g = torch.Generator().manual_seed(5)
     dt = torch.float32 if f32 else torch.bfloat16
-    T, top, E, n, k = 75, 2, 5, 40, 72
     x = torch.randn(T, k, generator=g).to(dt)
     w = (torch.randn(E, n, k, generator=g) / math.sqrt(k)).to(dt)
     ids = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(T)]).to(torch.int32)
