@@ -124,7 +124,8 @@ PROTOTYPES = {
                            _I, _I, _P]),
     "mv_latent_prep": (_I, [_P, _L, _P, _F, _P, _P, _L, _P, _L, _P, _L, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I,
                             _I, _I, _I, _P]),
-    "mv_latent_attn": (_I, [_P, _L, _P, _P, _L, _P, _P, _P, _I, _I, _P, _I, _I, _I, _I, _F, _I, _I, _P]),
+    "mv_latent_attn": (_I, [_P, _L, _P, _P, _L, _P, _P, _P, _I, _I, _P, _I, _I, _I, _I, _F, _I, _I, _P, _P, _P, _I, _I,
+                            _P]),
     "mv_moe_route": (_I, [_P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "mv_moe_plan": (_I, [_P, _P, _P, _P, _I, _I, _P]),
     "mv_moe_combine": (_I, [_P, _L, _P, _P, _P, _L, _P, _P, _L, _I, _I, _I, _P]),

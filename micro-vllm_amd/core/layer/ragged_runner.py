@@ -426,7 +426,7 @@ class RaggedRunner:
                         interleaved=first_kind)
         ops.linear_heads(q_plain, w["uk_t"], q_abs.view(T, H, R + r)[:, :, :R], H)
         lat = self._actbuf(T, H * R)
-        ops.latent_attn(q_abs, pages, lat, step, sink, H, R, r, float(m["scale"]), window)
+        ops.latent_attn(q_abs, pages, lat, step, sink, H, R, r, float(m["scale"]), window, tiled=self.tiled_attn)
         val = self._f32buf(T, H * dv)
         ops.linear_heads(lat, w["uv"], val.view(T, H, dv), H)
         a = self._actbuf(T, H * dv)

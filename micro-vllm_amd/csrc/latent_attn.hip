@@ -110,9 +110,13 @@ template <bool F32, int NW, int HG, int VC>
 __global__ __launch_bounds__(64 * NW) void latent_attn_kernel(const float* q, int64_t ldq, const void* cache_,
                                                               void* out_, int64_t ldo, LatentPages pr,
                                                               const float* sinks, int H, int R, int r, float scale,
-                                                              int window) {
+                                                              int window, const int* row_len, int max_len) {
     typedef typename ActL<F32>::T T_;
     extern __shared__ float lds[];
+    {   // rows of more than max_len tokens belong to the tile kernel
+        const int groups_ = (H + HG - 1) / HG;
+        if (max_len > 0 && row_len[pr.tok_row[blockIdx.x / groups_]] > max_len) return;
+    }
     const T_* cache = (const T_*)cache_;
     T_* out = (T_*)out_;
     const int d = R + r;
@@ -262,7 +266,8 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_kernel(const float* q, in
 
 template <bool F32, int NW, int HG, int VC>
 static int launch_latent_attn(const float* q, int64_t ldq, const void* cache, void* out, int64_t ldo, LatentPages pr,
-                              const float* sinks, int T, int H, int R, int r, float scale, int window, hipStream_t s) {
+                              const float* sinks, int T, int H, int R, int r, float scale, int window,
+                              const int* row_len, int max_len, hipStream_t s) {
     static LdsOptIn done;
     const size_t lds = (size_t)(HG * (R + r) + NW * HG * 64 + 2 * NW * HG + HG * R) * sizeof(float);
     if (lds > 150 * 1024) return MV_ERR_UNSUPPORTED;
@@ -273,17 +278,155 @@ static int launch_latent_attn(const float* q, int64_t ldq, const void* cache, vo
     }
     const int groups = (H + HG - 1) / HG;
     hipLaunchKernelGGL((latent_attn_kernel<F32, NW, HG, VC>), dim3((unsigned)((int64_t)T * groups)), dim3(64 * NW), lds, s,
-                       q, ldq, cache, out, ldo, pr, sinks, H, R, r, scale, window);
+                       q, ldq, cache, out, ldo, pr, sinks, H, R, r, scale, window, row_len, max_len);
     return check_launch();
 }
 
 template <bool F32, int NW, int HG>
 static int latent_attn_vc(const float* q, int64_t ldq, const void* cache, void* out, int64_t ldo, LatentPages pr,
-                          const float* sinks, int T, int H, int R, int r, float scale, int window, hipStream_t s) {
-    if (R <= 128) return launch_latent_attn<F32, NW, HG, 2>(q, ldq, cache, out, ldo, pr, sinks, T, H, R, r, scale, window, s);
-    if (R <= 256) return launch_latent_attn<F32, NW, HG, 4>(q, ldq, cache, out, ldo, pr, sinks, T, H, R, r, scale, window, s);
-    if (R <= 512) return launch_latent_attn<F32, NW, HG, 8>(q, ldq, cache, out, ldo, pr, sinks, T, H, R, r, scale, window, s);
+                          const float* sinks, int T, int H, int R, int r, float scale, int window, const int* row_len,
+                          int max_len, hipStream_t s) {
+    if (R <= 128) return launch_latent_attn<F32, NW, HG, 2>(q, ldq, cache, out, ldo, pr, sinks, T, H, R, r, scale, window, row_len, max_len, s);
+    if (R <= 256) return launch_latent_attn<F32, NW, HG, 4>(q, ldq, cache, out, ldo, pr, sinks, T, H, R, r, scale, window, row_len, max_len, s);
+    if (R <= 512) return launch_latent_attn<F32, NW, HG, 8>(q, ldq, cache, out, ldo, pr, sinks, T, H, R, r, scale, window, row_len, max_len, s);
     return MV_ERR_UNSUPPORTED;
+}
+
+// The same attention for a prompt's portion, bf16 pages of 64 tokens: one workgroup per (64 consecutive tokens of a
+// row, head), a wave per 16 of them.  A page is staged once in LDS and serves as keys (all R + r columns) and as
+// values (the first R).  q . k on v_mfma_f32_16x16x32_bf16 (q rounded to bf16 as the cached latents are), mask,
+// sink and softmax in fp32 per lane, P . V on v_mfma_f32_16x16x4_f32 with P staying fp32: a lane's score
+// accumulators S[key 16 nt + 4 (lane / 16) + j][query lane % 16] are exactly that instruction's second operand
+// for the four keys {16 nt + 4 g + j}, so P never leaves the registers.  KS = (R + r) / 32, CT = R / 16.
+typedef __attribute__((ext_vector_type(8))) __bf16 lt_bf16x8_t;
+
+template <int KS, int CT>
+__global__ __launch_bounds__(256) void latent_attn_tile_kernel(const float* q, int64_t ldq, const uint16_t* cache,
+                                                               uint16_t* out, int64_t ldo, LatentPages pr,
+                                                               const int* ch_start, const int* ch_len,
+                                                               const float* sinks, int H, float scale, int window) {
+    constexpr int D = KS * 32, DV = CT * 16, SK = D + 8;
+    extern __shared__ __attribute__((aligned(16))) uint16_t Ks[];   // [64][SK]
+    const int ch = blockIdx.x, h = blockIdx.y;
+    const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, r = lane & 15, qd = lane >> 4;
+    const int start = ch_start[ch], len = ch_len[ch];
+    const int* bt = pr.block_table + (int64_t)pr.tok_row[start] * pr.bt_stride;
+    const int p0 = pr.tok_pos[start];            // positions run on from here within the chunk
+    const int myq = 16 * wv + r;
+    const bool qok = myq < len;
+    const int qpos = p0 + myq;
+    const int win = window > 0 ? window : (1 << 30);
+    lt_bf16x8_t qf[KS];
+    {
+        const float* qp = q + (int64_t)(start + (qok ? myq : 0)) * ldq + (int64_t)h * D + 8 * qd;
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) {
+            const float4 a = *reinterpret_cast<const float4*>(qp + 32 * kk);
+            const float4 b = *reinterpret_cast<const float4*>(qp + 32 * kk + 4);
+            const uint4 pk = make_uint4(pack_bf16x2(a.x, a.y), pack_bf16x2(a.z, a.w), pack_bf16x2(b.x, b.y),
+                                        pack_bf16x2(b.z, b.w));
+            qf[kk] = __builtin_bit_cast(lt_bf16x8_t, pk);
+        }
+    }
+    float m = -INFINITY, l = 0.f;
+    f32x4_t o[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) o[ct] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    const int klo = p0 - win + 1 > 0 ? p0 - win + 1 : 0, khi = p0 + len - 1;
+    const int wq_lo = p0 + 16 * wv, wq_hi = wq_lo + 15;   // this wave's query positions
+    for (int kt = klo / 64; kt <= khi / 64; ++kt) {
+        const int kbase = kt * 64;
+        const int64_t pgrow = (int64_t)bt[kt] * 64;
+        __syncthreads();
+        for (int i = tid; i < 64 * (D / 8); i += 256) {
+            const int rr = i / (D / 8), cc = i % (D / 8);
+            st16(&Ks[rr * SK + cc * 8], ld16(cache + (pgrow + rr) * D + cc * 8));
+        }
+        __syncthreads();
+        if (kbase > wq_hi || kbase + 63 <= wq_lo - win) continue;   // nothing of this tile is visible to the wave
+        f32x4_t sc[4];
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) {
+            sc[nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kk = 0; kk < KS; ++kk) {
+                const lt_bf16x8_t kf = __builtin_bit_cast(lt_bf16x8_t, ld16(&Ks[(16 * nt + r) * SK + 32 * kk + 8 * qd]));
+                sc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[kk], sc[nt], 0, 0, 0);
+            }
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int kpos = kbase + 16 * nt + 4 * qd + j;
+                const bool ok = qok && kpos <= qpos && kpos > qpos - win;
+                const float v = ok ? sc[nt][j] * scale : -INFINITY;
+                sc[nt][j] = v;
+                mx = fmaxf(mx, v);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float mn = fmaxf(m, mx);
+        const float corr = m == -INFINITY ? 0.f : expf(m - mn);
+        float ps = 0.f;
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float pv = sc[nt][j] == -INFINITY ? 0.f : expf(sc[nt][j] - mn);
+                sc[nt][j] = pv;
+                ps += pv;
+            }
+        ps += __shfl_xor(ps, 16, 64);
+        ps += __shfl_xor(ps, 32, 64);
+        l = l * corr + ps;
+        m = mn;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) o[ct] *= corr;
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint16_t* vrow = &Ks[(16 * nt + 4 * qd + j) * SK + r];
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct)
+                    o[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(bf16_bits_to_f32(vrow[16 * ct]), sc[nt][j], o[ct], 0, 0, 0);
+            }
+    }
+    if (qok) {
+        // the sink joins the denominator as one more score without a value (a sink far above m: the output goes to zero)
+        const float inv = 1.0f / (sinks ? l + expf(sinks[h] - m) : l);
+        uint16_t* op = out + (int64_t)(start + myq) * ldo + (int64_t)h * DV + 4 * qd;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            uint2 w;
+            w.x = pack_bf16x2(o[ct][0] * inv, o[ct][1] * inv);
+            w.y = pack_bf16x2(o[ct][2] * inv, o[ct][3] * inv);
+            *reinterpret_cast<uint2*>(op + 16 * ct) = w;
+        }
+    }
+}
+
+template <int KS, int CT>
+static int launch_latent_tile(const float* q, int64_t ldq, const void* cache, void* out, int64_t ldo, LatentPages pr,
+                              const int* ch_start, const int* ch_len, int chunks, const float* sinks, int H,
+                              float scale, int window, hipStream_t s) {
+    static LdsOptIn done;
+    const size_t lds = (size_t)64 * (KS * 32 + 8) * sizeof(uint16_t);
+    const void* kern = (const void*)latent_attn_tile_kernel<KS, CT>;
+    if (lds > 48 * 1024) {
+        const int rc = ensure_dynamic_lds(kern, lds, done);
+        if (rc != MV_OK) return rc;
+    }
+    hipLaunchKernelGGL((latent_attn_tile_kernel<KS, CT>), dim3(chunks, H), dim3(256), lds, s, q, ldq,
+                       (const uint16_t*)cache, (uint16_t*)out, ldo, pr, ch_start, ch_len, sinks, H, scale, window);
+    return check_launch();
+}
+
+// the (latent width, rotated width) pairs the tile kernel is built for
+static bool latent_tile_shape(int R, int r) {
+    return (r == 32 || r == 64) && (R == 64 || R == 128 || R == 256 || R == 512) && (R + r) % 32 == 0;
 }
 
 }  // namespace mv
@@ -312,7 +455,8 @@ int mv_latent_prep(const float* dkv, int64_t ldkv, const float* w_norm, float ep
 
 int mv_latent_attn(const float* q_abs, int64_t ldq, const void* cache, void* out, int64_t ldo, const int32_t* tok_row,
                    const int32_t* tok_pos, const int32_t* block_table, int bt_stride, int page, const float* sinks,
-                   int tokens, int heads, int rank, int r, float scale, int window, int f32, mv_stream_t stream) {
+                   int tokens, int heads, int rank, int r, float scale, int window, int f32, const int32_t* row_len,
+                   const int32_t* ch_start, const int32_t* ch_len, int chunks, int max_len, mv_stream_t stream) {
     using namespace mv;
     if (tokens < 0 || heads <= 0 || rank <= 0 || r < 0 || page <= 0 || window < 0) return MV_ERR_INVALID_ARG;
     if (tokens == 0) return MV_OK;
@@ -321,18 +465,32 @@ int mv_latent_attn(const float* q_abs, int64_t ldq, const void* cache, void* out
         return MV_ERR_INVALID_ARG;
     const LatentPages pr{tok_row, tok_pos, block_table, bt_stride, page};
     hipStream_t s = (hipStream_t)stream;
+    // rows of more than max_len tokens (they are cut into the step's chunks) on the matrix cores where the shape fits
+    int plain_max = 0;
+    if (chunks > 0 && !f32 && page == 64 && heads <= 65535 && latent_tile_shape(rank, r) && row_len && ch_start &&
+        ch_len && max_len > 0 && ldq % 4 == 0 && ldo % 4 == 0 && aligned16(q_abs)) {
+        int rc = MV_ERR_UNSUPPORTED;
+#define MV_LT(R_, r_)                                                                                              \
+    if (rank == R_ && r == r_)                                                                                     \
+        rc = launch_latent_tile<(R_ + r_) / 32, R_ / 16>(q_abs, ldq, cache, out, ldo, pr, ch_start, ch_len, chunks, \
+                                                          sinks, heads, scale, window, s);
+        MV_LT(64, 32) MV_LT(64, 64) MV_LT(128, 32) MV_LT(128, 64) MV_LT(256, 32) MV_LT(256, 64) MV_LT(512, 32) MV_LT(512, 64)
+#undef MV_LT
+        if (rc != MV_OK) return rc;
+        plain_max = max_len;
+    }
     // few tokens (decoding): sixteen waves share a token's keys, so that the launch still fills the chip
     const bool few = (int64_t)tokens * ((heads + 3) / 4) < 2 * (int64_t)num_cus();
     // very few (a handful of decoded tokens): a workgroup per head rather than per four heads
     const bool alone = (int64_t)tokens * ((heads + 3) / 4) < 64;
     if (f32) {
-        if (alone) return latent_attn_vc<true, 16, 1>(q_abs, ldq, cache, out, ldo, pr, sinks, tokens, heads, rank, r, scale, window, s);
-        if (few) return latent_attn_vc<true, 16, 4>(q_abs, ldq, cache, out, ldo, pr, sinks, tokens, heads, rank, r, scale, window, s);
-        return latent_attn_vc<true, 4, 4>(q_abs, ldq, cache, out, ldo, pr, sinks, tokens, heads, rank, r, scale, window, s);
+        if (alone) return latent_attn_vc<true, 16, 1>(q_abs, ldq, cache, out, ldo, pr, sinks, tokens, heads, rank, r, scale, window, row_len, plain_max, s);
+        if (few) return latent_attn_vc<true, 16, 4>(q_abs, ldq, cache, out, ldo, pr, sinks, tokens, heads, rank, r, scale, window, row_len, plain_max, s);
+        return latent_attn_vc<true, 4, 4>(q_abs, ldq, cache, out, ldo, pr, sinks, tokens, heads, rank, r, scale, window, row_len, plain_max, s);
     }
-    if (alone) return latent_attn_vc<false, 16, 1>(q_abs, ldq, cache, out, ldo, pr, sinks, tokens, heads, rank, r, scale, window, s);
-    if (few) return latent_attn_vc<false, 16, 4>(q_abs, ldq, cache, out, ldo, pr, sinks, tokens, heads, rank, r, scale, window, s);
-    return latent_attn_vc<false, 4, 4>(q_abs, ldq, cache, out, ldo, pr, sinks, tokens, heads, rank, r, scale, window, s);
+    if (alone) return latent_attn_vc<false, 16, 1>(q_abs, ldq, cache, out, ldo, pr, sinks, tokens, heads, rank, r, scale, window, row_len, plain_max, s);
+    if (few) return latent_attn_vc<false, 16, 4>(q_abs, ldq, cache, out, ldo, pr, sinks, tokens, heads, rank, r, scale, window, row_len, plain_max, s);
+    return latent_attn_vc<false, 4, 4>(q_abs, ldq, cache, out, ldo, pr, sinks, tokens, heads, rank, r, scale, window, row_len, plain_max, s);
 }
 
 }  // extern "C"

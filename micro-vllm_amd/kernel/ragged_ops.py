@@ -408,8 +408,11 @@ def latent_prep(dkv, w_norm, eps: float, cache, q, q_plain, q_abs, inv_freq, ste
         int(interleaved), _is_f32(cache), nv.stream_ptr()))
 
 
-def latent_attn(q_abs, cache, out, step, sinks, heads: int, rank: int, r: int, scale: float, window: int):
-    """out [T, heads*rank] in the activation type: weighted sums of the cached latents.  window 0: causal."""
+def latent_attn(q_abs, cache, out, step, sinks, heads: int, rank: int, r: int, scale: float, window: int,
+                tiled: bool = True):
+    """out [T, heads*rank] in the activation type: weighted sums of the cached latents.  window 0: causal.
+    `tiled`: rows of more than SCAN_SEQ_MAX tokens go to the matrix-core kernel where it applies (bf16, the
+    shapes it is built for); False keeps every token on the plain kernel."""
     tokens = q_abs.shape[0]
     assert q_abs.shape == (tokens, heads * (rank + r)) and out.shape == (tokens, heads * rank)
     assert cache.is_contiguous() and cache.shape[1:] == (step.page, rank + r) and int(step.max_page) < cache.shape[0]
@@ -419,7 +422,9 @@ def latent_attn(q_abs, cache, out, step, sinks, heads: int, rank: int, r: int, s
         _f32(q_abs).data_ptr(), _ld(q_abs), cache.data_ptr(), out.data_ptr(), _ld(out), step.tok_row.data_ptr(),
         step.tok_pos.data_ptr(), step.block_table.data_ptr(), step.block_table.stride(0), step.page,
         None if sinks is None else _f32(sinks).data_ptr(), tokens, heads, rank, r, float(scale), int(window),
-        _is_f32(cache), nv.stream_ptr()))
+        _is_f32(cache), step.row_len.data_ptr(), step.ch_start.data_ptr() if step.n_chunks else None,
+        step.ch_len.data_ptr() if step.n_chunks else None, step.n_chunks if tiled else 0, SCAN_SEQ_MAX,
+        nv.stream_ptr()))
 
 
 def moe_route(h, w_router, w_shared_gate, ids, weights, shared_gate):
