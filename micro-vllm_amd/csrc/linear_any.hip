@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256) void linear_any_bf16_kernel(
 // The same product on a 128 x 128 tile for launches with many rows: four waves as 2 x 2, each 64 x 64 (sixteen
 // accumulator tiles), so that a k-step of 32 costs a wave eight LDS reads for sixteen matrix instructions
 // instead of five for four.  Same order of the sums over k as the 64 x 64 form: the results are equal bit for bit.
-constexpr int kLbBM = 128, kLbBN = 128;
+constexpr int kLbBM = 128, kLbBN = 128, kLbBK = 64, kLbPad = 72;   // LDS row = 72 bf16 = 144 bytes
 
 __global__ __launch_bounds__(256) void linear_any_bf16_big_kernel(
     const uint16_t* __restrict__ x, int64_t ldx, const uint16_t* __restrict__ w, int64_t ldw,
@@ -109,12 +109,12 @@ __global__ __launch_bounds__(256) void linear_any_bf16_big_kernel(
     x += blockIdx.z * zx;
     w += blockIdx.z * zw;
     y += blockIdx.z * zy;
-    __shared__ __attribute__((aligned(16))) uint16_t xs[kLbBM][kLaPad];
-    __shared__ __attribute__((aligned(16))) uint16_t ws[kLbBN][kLaPad];
+    __shared__ __attribute__((aligned(16))) uint16_t xs[kLbBM][kLbPad];
+    __shared__ __attribute__((aligned(16))) uint16_t ws[kLbBN][kLbPad];
     const int m0 = blockIdx.y * kLbBM, n0 = blockIdx.x * kLbBN;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, q = lane >> 4;
     const int wm = wave >> 1, wn = wave & 1;
-    const int lrow = tid >> 2, lcol = (tid & 3) * 8;
+    const int lrow = tid >> 3, lcol = (tid & 7) * 8;   // a thread stages rows lrow + 32 u, eight values at lcol
     int64_t y0 = 0;
     if (sg.seg) {
         y0 = sg.seg[blockIdx.z];
@@ -122,10 +122,10 @@ __global__ __launch_bounds__(256) void linear_any_bf16_big_kernel(
         if (m0 >= M) return;
         y += y0 * ldy;
     }
-    const uint16_t* xp[2];
+    const uint16_t* xp[4];
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-        const int mr = m0 + lrow + 64 * u;
+    for (int u = 0; u < 4; ++u) {
+        const int mr = m0 + lrow + 32 * u;
         const int64_t xrow = mr < M ? (sg.src ? sg.src[y0 + mr] / sg.src_div : y0 + mr) : 0;
         xp[u] = x + xrow * ldx;
     }
@@ -134,38 +134,41 @@ __global__ __launch_bounds__(256) void linear_any_bf16_big_kernel(
     for (int a = 0; a < 4; ++a)
 #pragma unroll
         for (int b = 0; b < 4; ++b) acc[a][b] = f32x4_t{0, 0, 0, 0};
-    uint4 xr[2], wr[2];
+    uint4 xr[4], wr[4];
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-        xr[u] = la_load8(xp[u], ldx, 0, m0 + lrow + 64 * u < M ? 1 : 0, lcol, K, vec_x);
-        wr[u] = la_load8(w, ldw, n0 + lrow + 64 * u, N, lcol, K, vec_w);
+    for (int u = 0; u < 4; ++u) {
+        xr[u] = la_load8(xp[u], ldx, 0, m0 + lrow + 32 * u < M ? 1 : 0, lcol, K, vec_x);
+        wr[u] = la_load8(w, ldw, n0 + lrow + 32 * u, N, lcol, K, vec_w);
     }
-    for (int k0 = 0; k0 < K; k0 += kLaBK) {
+    for (int k0 = 0; k0 < K; k0 += kLbBK) {
         __syncthreads();
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            st16(&xs[lrow + 64 * u][lcol], xr[u]);
-            st16(&ws[lrow + 64 * u][lcol], wr[u]);
+        for (int u = 0; u < 4; ++u) {
+            st16(&xs[lrow + 32 * u][lcol], xr[u]);
+            st16(&ws[lrow + 32 * u][lcol], wr[u]);
         }
         __syncthreads();
-        if (k0 + kLaBK < K) {
+        if (k0 + kLbBK < K) {
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                xr[u] = la_load8(xp[u], ldx, 0, m0 + lrow + 64 * u < M ? 1 : 0, k0 + kLaBK + lcol, K, vec_x);
-                wr[u] = la_load8(w, ldw, n0 + lrow + 64 * u, N, k0 + kLaBK + lcol, K, vec_w);
+            for (int u = 0; u < 4; ++u) {
+                xr[u] = la_load8(xp[u], ldx, 0, m0 + lrow + 32 * u < M ? 1 : 0, k0 + kLbBK + lcol, K, vec_x);
+                wr[u] = la_load8(w, ldw, n0 + lrow + 32 * u, N, k0 + kLbBK + lcol, K, vec_w);
             }
         }
-        la_bf16x8_t wf[4], xf[4];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            wf[t] = __builtin_bit_cast(la_bf16x8_t, ld16(&ws[wn * 64 + t * 16 + r][q * 8]));
-            xf[t] = __builtin_bit_cast(la_bf16x8_t, ld16(&xs[wm * 64 + t * 16 + r][q * 8]));
+        for (int ks = 0; ks < kLbBK; ks += 32) {   // two steps of 32, in ascending k as the narrow tile takes them
+            la_bf16x8_t wf[4], xf[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                wf[t] = __builtin_bit_cast(la_bf16x8_t, ld16(&ws[wn * 64 + t * 16 + r][ks + q * 8]));
+                xf[t] = __builtin_bit_cast(la_bf16x8_t, ld16(&xs[wm * 64 + t * 16 + r][ks + q * 8]));
+            }
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+                for (int mt = 0; mt < 4; ++mt)
+                    acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[nt], xf[mt], acc[nt][mt], 0, 0, 0);
         }
-#pragma unroll
-        for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-            for (int mt = 0; mt < 4; ++mt)
-                acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[nt], xf[mt], acc[nt][mt], 0, 0, 0);
     }
     // acc[nt][mt][j] = C[n = n0 + 64 wn + 16 nt + 4 q + j][m = m0 + 64 wm + 16 mt + r]
 #pragma unroll
@@ -173,12 +176,17 @@ __global__ __launch_bounds__(256) void linear_any_bf16_big_kernel(
         const int m = m0 + wm * 64 + mt * 16 + r;
         if (m >= M) continue;
 #pragma unroll
-        for (int nt = 0; nt < 4; ++nt)
+        for (int nt = 0; nt < 4; ++nt) {
+            const int n = n0 + wn * 64 + nt * 16 + q * 4;
+            float* dst = y + (int64_t)m * ldy + n;
+            if (n + 3 < N && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+                *reinterpret_cast<float4*>(dst) = make_float4(acc[nt][mt][0], acc[nt][mt][1], acc[nt][mt][2], acc[nt][mt][3]);
+            } else {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int n = n0 + wn * 64 + nt * 16 + q * 4 + j;
-                if (n < N) y[(int64_t)m * ldy + n] = acc[nt][mt][j];
+                for (int j = 0; j < 4; ++j)
+                    if (n + j < N) dst[j] = acc[nt][mt][j];
             }
+        }
     }
 }
 
