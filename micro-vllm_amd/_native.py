@@ -159,6 +159,9 @@ def lib():
     the entry points it lacks raise AttributeError when they are first asked for."""
     global _lib
     if _lib is None:
+        # torch first: its own copy of the HIP runtime must be the one this library binds to, or the process ends
+        # up with two runtimes of which the second sees no device
+        import torch  # noqa: F401
         path, whole = LIB_PATH, True
         if not os.path.exists(path):
             parts = [] if os.environ.get("MVLLM_LIB") else _part_libraries()

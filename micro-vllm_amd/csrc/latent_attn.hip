@@ -289,6 +289,7 @@ static int latent_attn_vc(const float* q, int64_t ldq, const void* cache, void* 
     if (R <= 128) return launch_latent_attn<F32, NW, HG, 2>(q, ldq, cache, out, ldo, pr, sinks, T, H, R, r, scale, window, row_len, max_len, s);
     if (R <= 256) return launch_latent_attn<F32, NW, HG, 4>(q, ldq, cache, out, ldo, pr, sinks, T, H, R, r, scale, window, row_len, max_len, s);
     if (R <= 512) return launch_latent_attn<F32, NW, HG, 8>(q, ldq, cache, out, ldo, pr, sinks, T, H, R, r, scale, window, row_len, max_len, s);
+    if (R <= 1024) return launch_latent_attn<F32, NW, HG, 16>(q, ldq, cache, out, ldo, pr, sinks, T, H, R, r, scale, window, row_len, max_len, s);
     return MV_ERR_UNSUPPORTED;
 }
 
