@@ -574,9 +574,11 @@ int mv_dyt_shift(const float* x, int64_t ldx, const float* w, const float* b, co
 /* out[r,:] = act( tanh(alpha x[idx[r],:]) w + b ); idx == NULL: row r itself. */
 int mv_dyt_gather(const float* x, int64_t ldx, const int32_t* idx, const float* w, const float* b, const float* alpha,
                   void* out, int64_t ldo, int rows, int n, int f32, mv_stream_t stream);
-/* x += tanh(alpha y) w + b; h = act(x) unless h == NULL. */
+/* x += tanh(alpha y) w + b; h = act(x) unless h == NULL; with w2 != NULL h = act( tanh(alpha2 x) w2 + b2 ), the next
+ * sublayer's norm of the new x. */
 int mv_dyt_residual(const float* y, int64_t ldy, const float* w, const float* b, const float* alpha, float* x,
-                    int64_t ldx, void* h, int64_t ldh, int rows, int n, int f32, mv_stream_t stream);
+                    int64_t ldx, void* h, int64_t ldh, const float* w2, const float* b2, const float* alpha2, int rows,
+                    int n, int f32, mv_stream_t stream);
 /* x += y / sqrt(mean(y^2) + eps) * w (plain weight); h = act(x) unless h == NULL. */
 int mv_unitnorm_residual(const float* y, int64_t ldy, const float* w, float eps, float* x, int64_t ldx, void* h,
                          int64_t ldh, int rows, int n, int f32, mv_stream_t stream);
@@ -651,10 +653,12 @@ int mv_moe_route(const void* h, int64_t ldh, const float* w_router, const float*
 /* (token, choice) pairs sorted by expert: seg [experts + 1], order [pairs] (pair in each row), place [pairs]. */
 int mv_moe_plan(const int32_t* ids, int32_t* seg, int32_t* order, int32_t* place, int pairs, int experts,
                 mv_stream_t stream);
-/* y_t = sum_k weights[t,k] * expert_out[place[t*top+k]] (+ shared_gate[t] * shared_out[t]). */
+/* s_t = sum_k weights[t,k] * expert_out[place[t*top+k]] (+ shared_gate[t] * shared_out[t]).  norm_w == NULL: y = s.
+ * Else y is the residual stream: y += tanh(norm_alpha s) norm_w + norm_b, and h (optional) = act(y). */
 int mv_moe_combine(const float* expert_out, int64_t lde, const int32_t* place, const float* weights,
-                   const float* shared_out, int64_t lds, const float* shared_gate, float* y, int64_t ldy, int tokens,
-                   int n, int top, mv_stream_t stream);
+                   const float* shared_out, int64_t lds, const float* shared_gate, float* y, int64_t ldy,
+                   const float* norm_w, const float* norm_b, const float* norm_alpha, void* h, int64_t ldh, int tokens,
+                   int n, int top, int f32, mv_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -111,7 +111,7 @@ PROTOTYPES = {
                             _P, _P, _P, _I, _I, _P]),
     "mv_dyt_shift": (_I, [_P, _L, _P, _P, _P, _P, _P, _P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _P]),
     "mv_dyt_gather": (_I, [_P, _L, _P, _P, _P, _P, _P, _L, _I, _I, _I, _P]),
-    "mv_dyt_residual": (_I, [_P, _L, _P, _P, _P, _P, _L, _P, _L, _I, _I, _I, _P]),
+    "mv_dyt_residual": (_I, [_P, _L, _P, _P, _P, _P, _L, _P, _L, _P, _P, _P, _I, _I, _I, _P]),
     "mv_unitnorm_residual": (_I, [_P, _L, _P, _F, _P, _L, _P, _L, _I, _I, _I, _P]),
     "mv_rmsnorm_rows": (_I, [_P, _L, _I, _P, _F, _P, _L, _I, _I, _I, _P]),
     "mv_gelu_gate_rows": (_I, [_P, _L, _P, _L, _I, _P, _I, _P, _L, _I, _I, _I, _P]),
@@ -128,7 +128,7 @@ PROTOTYPES = {
                             _P]),
     "mv_moe_route": (_I, [_P, _L, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "mv_moe_plan": (_I, [_P, _P, _P, _P, _I, _I, _P]),
-    "mv_moe_combine": (_I, [_P, _L, _P, _P, _P, _L, _P, _P, _L, _I, _I, _I, _P]),
+    "mv_moe_combine": (_I, [_P, _L, _P, _P, _P, _L, _P, _P, _L, _P, _P, _P, _P, _L, _I, _I, _I, _I, _P]),
     "mv_graph_begin_capture": (_I, [_P]),
     "mv_graph_end_capture": (_I, [_P, ctypes.POINTER(c_void_p)]),
     "mv_graph_launch": (_I, [_P, _P]),

@@ -29,9 +29,10 @@ Per layer (Fagunex; norms are Dynamic Tanh, before and after each sublayer):
             space -> attention over the cached latents (window / causal, sink or none) -> per-head value
             up-projection -> (sigmoid gate,) cast -> out-projection
   then      x += norm1b(mixer output)
-  moe       norm2 -> router (fp32, top-k, softmax over the chosen, shared expert's sigmoid) -> (token, choice)
-            pairs sorted by expert -> gate|up by segment -> SiLU-gate -> down by segment; shared expert
-            gate|up -> SiLU-gate -> down; weighted sum -> x += norm2b(sum)
+  moe       (norm2 comes out of the launch that adds the mixer) -> router (fp32, top-k, softmax over the chosen,
+            shared expert's sigmoid) -> (token, choice) pairs sorted by expert -> gate|up by segment -> SiLU-gate ->
+            down by segment; shared expert gate|up -> SiLU-gate -> down; weighted sum, norm2b and the residual sum
+            in one launch
   side      gate projection of x -> gelu_tanh * slice of the second embedding -> projection ->
             x += unit-RMS * weight
 """
@@ -382,12 +383,14 @@ class RaggedRunner:
         else:
             y = self._latent_attention(li, w, layer["mixer"], h, step, cache, layer["type"] == "latent_attention")
         mlp = layer.get("mlp")
-        # the copy of x in the activation type is what the side input's gate reads when no feed-forward follows
-        ops.dyt_residual(y, w["norm1b"], x, h if (not mlp and cfg.side_dim) else None)
         if mlp:
-            ops.dyt_gather(x, None, w["norm2"], h)
-            y = self._moe(w, mlp, h, T)
-            ops.dyt_residual(y, w["norm2b"], x, h if cfg.side_dim else None)
+            # the norm after the mixer, the residual sum and the norm before the feed-forward in one launch; the
+            # experts' weighted sum goes through the norm after the feed-forward straight into the stream
+            ops.dyt_residual(y, w["norm1b"], x, h, next_norm=w["norm2"])
+            self._moe(w, mlp, h, T, x, w["norm2b"], h if cfg.side_dim else None)
+        else:
+            # the copy of x in the activation type is what the side input's gate reads
+            ops.dyt_residual(y, w["norm1b"], x, h if cfg.side_dim else None)
         if cfg.side_dim:
             a = w["side_gate"](h, self._f32buf(T, cfg.side_dim))
             g = self._actbuf(T, cfg.side_dim)
@@ -433,7 +436,7 @@ class RaggedRunner:
         ops.sigmoid_gate(val, gate, a)
         return w["w_o"](a, self._f32buf(T, self.width))
 
-    def _moe(self, w, mlp, h, T):
+    def _moe(self, w, mlp, h, T, x, norm_after, h_out):
         E, top, ff = int(mlp["router"]["experts"]), int(mlp["router"]["top"]), int(mlp["expert"]["ff"])
         shared = mlp.get("shared")
         ids = self._i32buf(T * top).view(T, top)
@@ -451,6 +454,4 @@ class RaggedRunner:
             s_act = self._actbuf(T, sf)
             ops.silu_mul(w["s_gu"](h, self._f32buf(T, 2 * sf)), s_act)
             s_out = w["s_down"](s_act, self._f32buf(T, self.width))
-        y = self._f32buf(T, self.width)
-        ops.moe_combine(down, place, wts, s_out, sgate, y)
-        return y
+        ops.moe_combine(down, place, wts, s_out, sgate, x, norm=norm_after, h=h_out)

@@ -8,7 +8,8 @@
 //                rows, order[i] the pair (token * top + choice) in row i, place[pair] its row.  The order inside
 //                an expert is whatever the atomics give; no result depends on it, since a row's products do
 //                not depend on the other rows (mv_linear_segments)
-//   moe_combine  y_t = sum_k weight[t,k] * expert_out[place[t,k]] (+ factor_t * shared_out_t)
+//   moe_combine  y_t = sum_k weight[t,k] * expert_out[place[t,k]] (+ factor_t * shared_out_t); with a norm given
+//                the sum goes through it straight into the stream: y += tanh(alpha sum) w + b
 // The experts' products themselves are mv_linear_segments (linear_any.hip) with a SiLU-gate between them.
 #include "common.h"
 
@@ -96,10 +97,14 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* ids, int* seg
     }
 }
 
+// norm_w != NULL: the sum does not go to y but through the norm after the sublayer into the stream,
+// x += tanh(alpha sum) w + b, and h (optional) = x in the activation type
+template <bool F32>
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* eo, int64_t lde, const int* place,
                                                           const float* wts, const float* so, int64_t lds_,
                                                           const float* shared_gate, float* y, int64_t ldy, int n,
-                                                          int top) {
+                                                          int top, const float* norm_w, const float* norm_b,
+                                                          const float* norm_alpha, void* h_, int64_t ldh) {
     const int t = blockIdx.x;
     int rows[kMaxTop];
     float w[kMaxTop];
@@ -113,6 +118,13 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* eo, int64
         float acc = 0.f;
         for (int k = 0; k < top; ++k) acc = fmaf(w[k], eo[(int64_t)rows[k] * lde + c], acc);
         if (so) acc = fmaf(g, so[(int64_t)t * lds_ + c], acc);
+        if (norm_w) {
+            acc = y[(int64_t)t * ldy + c] + fmaf(tanhf(norm_alpha[0] * acc), norm_w[c], norm_b[c]);
+            if (h_) {
+                if (F32) ((float*)h_)[(int64_t)t * ldh + c] = acc;
+                else ((uint16_t*)h_)[(int64_t)t * ldh + c] = (uint16_t)f32_to_bf16_bits(acc);
+            }
+        }
         y[(int64_t)t * ldy + c] = acc;
     }
 }
@@ -146,16 +158,19 @@ int mv_moe_plan(const int32_t* ids, int32_t* seg, int32_t* order, int32_t* place
 }
 
 int mv_moe_combine(const float* expert_out, int64_t lde, const int32_t* place, const float* weights,
-                   const float* shared_out, int64_t lds, const float* shared_gate, float* y, int64_t ldy, int tokens,
-                   int n, int top, mv_stream_t stream) {
+                   const float* shared_out, int64_t lds, const float* shared_gate, float* y, int64_t ldy,
+                   const float* norm_w, const float* norm_b, const float* norm_alpha, void* h, int64_t ldh, int tokens,
+                   int n, int top, int f32, mv_stream_t stream) {
     using namespace mv;
     if (tokens < 0 || n <= 0 || top <= 0 || top > kMaxTop) return MV_ERR_INVALID_ARG;
     if (tokens == 0) return MV_OK;
     if (!expert_out || !place || !weights || !y || (shared_out && !shared_gate) || lde < n || ldy < n ||
         (shared_out && lds < n))
         return MV_ERR_INVALID_ARG;
-    hipLaunchKernelGGL(moe_combine_kernel, dim3(tokens, (n + 255) / 256), dim3(256), 0, (hipStream_t)stream, expert_out, lde, place,
-                       weights, shared_out, lds, shared_gate, y, ldy, n, top);
+    if (norm_w ? (!norm_b || !norm_alpha || (h && ldh < n)) : h != nullptr) return MV_ERR_INVALID_ARG;
+    const dim3 grid(tokens, (n + 255) / 256);
+    if (f32) hipLaunchKernelGGL(moe_combine_kernel<true>, grid, dim3(256), 0, (hipStream_t)stream, expert_out, lde, place, weights, shared_out, lds, shared_gate, y, ldy, n, top, norm_w, norm_b, norm_alpha, h, ldh);
+    else hipLaunchKernelGGL(moe_combine_kernel<false>, grid, dim3(256), 0, (hipStream_t)stream, expert_out, lde, place, weights, shared_out, lds, shared_gate, y, ldy, n, top, norm_w, norm_b, norm_alpha, h, ldh);
     return check_launch();
 }
 

@@ -12,7 +12,7 @@
 //   dyt_shift:           n = tanh(alpha x) w + b (a norm without statistics); h_t = act( n_t + (n_(t-1) - n_t) mix ),
 //                        the last n of every row kept per state slot for the row's next step
 //   dyt_gather:          out = act( tanh(alpha x[idx]) w + b )
-//   dyt_residual:        x += tanh(alpha y) w + b; h = act(x)
+//   dyt_residual:        x += tanh(alpha y) w + b; h = act(x), or act of the next sublayer's norm of x
 //   unitnorm_residual:   x += y / sqrt(mean(y^2) + eps) * w; h = act(x)     (plain weight)
 //   rmsnorm_rows:        out = act( v / sqrt(mean(v^2) + eps) * w )         (plain weight, rows of any stride)
 //   gelu_gate_rows:      out = act( gelu_tanh(a) * table[id][off .. off+n) )
@@ -156,10 +156,12 @@ __global__ __launch_bounds__(256) void dyt_gather_kernel(const float* x, int64_t
     if (c < n) Act<F32>::st(out + (int64_t)row * ldo + c, fmaf(tanhf(al * a[c]), w[c], b[c]));
 }
 
+// w2 != NULL: h receives the NEXT sublayer's norm of the new x, tanh(alpha2 x) w2 + b2, instead of x itself
 template <bool F32>
 __global__ __launch_bounds__(256) void dyt_residual_kernel(const float* y, int64_t ldy, const float* w, const float* b,
                                                            const float* alpha, float* x, int64_t ldx, void* h_,
-                                                           int64_t ldh, int n) {
+                                                           int64_t ldh, int n, const float* w2, const float* b2,
+                                                           const float* alpha2) {
     typedef typename Act<F32>::T T;
     T* h = (T*)h_;
     const int row = blockIdx.x;
@@ -168,7 +170,7 @@ __global__ __launch_bounds__(256) void dyt_residual_kernel(const float* y, int64
     if (c < n) {
         const float s = x[(int64_t)row * ldx + c] + fmaf(tanhf(al * y[(int64_t)row * ldy + c]), w[c], b[c]);
         x[(int64_t)row * ldx + c] = s;
-        if (h) Act<F32>::st(h + (int64_t)row * ldh + c, s);
+        if (h) Act<F32>::st(h + (int64_t)row * ldh + c, w2 ? fmaf(tanhf(alpha2[0] * s), w2[c], b2[c]) : s);
     }
 }
 
@@ -356,13 +358,15 @@ int mv_dyt_gather(const float* x, int64_t ldx, const int32_t* idx, const float* 
 }
 
 int mv_dyt_residual(const float* y, int64_t ldy, const float* w, const float* b, const float* alpha, float* x,
-                    int64_t ldx, void* h, int64_t ldh, int rows, int n, int f32, mv_stream_t stream) {
+                    int64_t ldx, void* h, int64_t ldh, const float* w2, const float* b2, const float* alpha2, int rows,
+                    int n, int f32, mv_stream_t stream) {
     using namespace mv;
     if (rows < 0 || n <= 0) return MV_ERR_INVALID_ARG;
     if (rows == 0) return MV_OK;
     if (!y || !w || !b || !alpha || !x || ldy < n || ldx < n || (h && ldh < n)) return MV_ERR_INVALID_ARG;
+    if (w2 && (!b2 || !alpha2 || !h)) return MV_ERR_INVALID_ARG;
     hipStream_t s = (hipStream_t)stream;
-    MV_F32_LAUNCH(dyt_residual_kernel, dim3(rows, (n + 255) / 256), y, ldy, w, b, alpha, x, ldx, h, ldh, n);
+    MV_F32_LAUNCH(dyt_residual_kernel, dim3(rows, (n + 255) / 256), y, ldy, w, b, alpha, x, ldx, h, ldh, n, w2, b2, alpha2);
     return check_launch();
 }
 

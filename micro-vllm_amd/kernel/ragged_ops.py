@@ -273,14 +273,17 @@ def dyt_gather(x, idx, norm, out):
         rows, n, _is_f32(out), nv.stream_ptr()))
 
 
-def dyt_residual(y, norm, x, h=None, f32: bool = False):
-    """x += tanh(alpha y) w + b; h (optional) = x in the activation type."""
+def dyt_residual(y, norm, x, h=None, next_norm=None):
+    """x += tanh(alpha y) w + b; h (optional) = x in the activation type, or with `next_norm` that norm of the new x
+    (what the next sublayer reads)."""
     rows, n = x.shape
     assert y.shape == (rows, n) and norm[0].numel() == n and (h is None or h.shape == (rows, n))
+    assert next_norm is None or (h is not None and next_norm[0].numel() == n)
     w, b, a = _dyt(norm)
+    w2, b2, a2 = _dyt(next_norm) if next_norm is not None else (None, None, None)
     nv.check("mv_dyt_residual", nv.lib().mv_dyt_residual(
         _f32(y).data_ptr(), _ld(y), w, b, a, _f32(x).data_ptr(), _ld(x), None if h is None else h.data_ptr(),
-        0 if h is None else _ld(h), rows, n, int(f32) if h is None else _is_f32(h), nv.stream_ptr()))
+        0 if h is None else _ld(h), w2, b2, a2, rows, n, 0 if h is None else _is_f32(h), nv.stream_ptr()))
 
 
 def unitnorm_residual(y, w, eps: float, x, h=None):
@@ -449,13 +452,19 @@ def moe_plan(ids, seg, order, place, experts: int):
         nv.stream_ptr()))
 
 
-def moe_combine(expert_out, place, weights, shared_out, shared_gate, y):
+def moe_combine(expert_out, place, weights, shared_out, shared_gate, y, norm=None, h=None):
+    """y = the weighted sum of each token's experts (+ shared_gate * shared_out).  With `norm` y is the residual
+    stream and receives the sum through that norm, y += tanh(alpha sum) w + b; h (optional) = y in the activation
+    type."""
     tokens, n = y.shape
     top = weights.shape[1]
     assert expert_out.shape == (tokens * top, n) and place.numel() == tokens * top and weights.is_contiguous()
     assert shared_out is None or (shared_out.shape == (tokens, n) and shared_gate.numel() == tokens)
+    assert h is None or (norm is not None and h.shape == (tokens, n))
+    w, b, a = _dyt(norm) if norm is not None else (None, None, None)
     nv.check("mv_moe_combine", nv.lib().mv_moe_combine(
         _f32(expert_out).data_ptr(), _ld(expert_out), _i32(place).data_ptr(), _f32(weights).data_ptr(),
         None if shared_out is None else _f32(shared_out).data_ptr(), 0 if shared_out is None else _ld(shared_out),
-        None if shared_out is None else _f32(shared_gate).data_ptr(), _f32(y).data_ptr(), _ld(y), tokens, n, top,
-        nv.stream_ptr()))
+        None if shared_out is None else _f32(shared_gate).data_ptr(), _f32(y).data_ptr(), _ld(y), w, b, a,
+        None if h is None else h.data_ptr(), 0 if h is None else _ld(h), tokens, n, top,
+        0 if h is None else _is_f32(h), nv.stream_ptr()))

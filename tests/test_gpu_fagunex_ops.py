@@ -126,6 +126,13 @@ def test_rowwise_steps(ops, f32):
     assert (o.cpu().double() - y.double() * torch.sigmoid(gt.double())).abs().max().item() < tol
     ops.sigmoid_gate(y.to(DEV), None, o)
     assert torch.equal(o.cpu(), y.to(dt))
+    # the residual step that also hands out the next sublayer's norm of the new x
+    norm2 = dyt(n, g)
+    x1 = xd.cpu().double()
+    ops.dyt_residual(y.to(DEV), dev(norm), xd, h, next_norm=dev(norm2))
+    x2 = x1 + ref.dynamic_tanh(y.double(), *nd)
+    assert (xd.cpu().double() - x2).abs().max().item() < 2e-5
+    assert (h.cpu().double() - ref.dynamic_tanh(x2, *[t.double() for t in norm2])).abs().max().item() < tol
 
 
 @pytest.mark.parametrize("f32", [False, True])
@@ -437,3 +444,10 @@ def test_routed_experts(ops, f32, E, top, shared):
     y = torch.empty(T, W, device=DEV)
     ops.moe_combine(down, place, wts, s_out, sg if shared else None, y)
     assert (y.cpu().double() - want).abs().max().item() < (3e-5 if f32 else 4e-2)
+    # the same sum sent through a norm into a residual stream, with the stream's copy in the activation type
+    norm = dyt(W, g)
+    x0 = torch.randn(T, W, generator=g)
+    x, hx = x0.to(DEV), torch.empty(T, W, dtype=dt, device=DEV)
+    ops.moe_combine(down, place, wts, s_out, sg if shared else None, x, norm=dev(norm), h=hx)
+    fused = x0.double() + ref.dynamic_tanh(y.cpu().double(), *[t.double() for t in norm])
+    assert (x.cpu().double() - fused).abs().max().item() < 1e-5 and torch.equal(hx.cpu(), x.cpu().to(dt))
