@@ -967,18 +967,22 @@ int mv_scan_gated(const float* q, int64_t ldq, const float* f, int64_t ldf, cons
     a.r = StepRows{nullptr, nullptr, row_start, row_len, row_ctx, row_slot};
     a.H = heads; a.n = n; a.p = p; a.max_len = chunks > 0 ? max_len : 0;
     a.ch_start = nullptr; a.ch_len = nullptr; a.ds = nullptr;
-    a.pt = p % 64 == 0 ? 64 : (p % 32 == 0 ? 32 : 16);
-    while (a.pt > 16 && (n + 256 / a.pt - 1) / (256 / a.pt) > 64) a.pt /= 2;
-    const int ns = 256 / a.pt, npt = (n + ns - 1) / ns;
-    if (npt > 64) return MV_ERR_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
-    const int tiles = (p + a.pt - 1) / a.pt;
     // rows of up to max_len tokens (all rows when nothing is cut into chunks): token by token from the slot's state
     for (int pass = 0; pass < (chunks > 0 ? 2 : 1); ++pass) {
         if (pass == 1) {
             a.ch_start = ch_start; a.ch_len = ch_len; a.ds = ds;
         }
-        const dim3 grid(tiles, heads, pass == 0 ? rows : chunks);
+        const int units = pass == 0 ? rows : chunks;
+        a.pt = p % 64 == 0 ? 64 : (p % 32 == 0 ? 32 : 16);
+        // a state too tall for 64 rows a thread: narrower column tiles leave more threads to share its rows; so do
+        // launches that would not fill the chip otherwise (a few decoded tokens: the step is the state's traffic)
+        while (a.pt > 16 && ((n + 256 / a.pt - 1) / (256 / a.pt) > 64 ||
+                             (int64_t)((p + a.pt - 1) / a.pt) * heads * units < 2 * (int64_t)num_cus()))
+            a.pt /= 2;
+        const int ns = 256 / a.pt, npt = (n + ns - 1) / ns;
+        if (npt > 64) return MV_ERR_UNSUPPORTED;
+        const dim3 grid((p + a.pt - 1) / a.pt, heads, units);
         if (npt <= 4) hipLaunchKernelGGL((scan_outer_kernel<4, true>), grid, dim3(256), 0, s, a);
         else if (npt <= 16) hipLaunchKernelGGL((scan_outer_kernel<16, true>), grid, dim3(256), 0, s, a);
         else hipLaunchKernelGGL((scan_outer_kernel<64, true>), grid, dim3(256), 0, s, a);
